@@ -417,3 +417,162 @@ class ZiferaxConfig:
     @property
     def num_hidden_layers(self) -> int:
         return len(self.layers)
+
+
+@dataclass(frozen=True)
+class RotaryScaling:
+    """Frequencies stretched by wavelength: pairs that turn fewer than ``slow`` times over ``original`` positions
+    have their frequency divided by ``factor``, pairs that turn more than ``fast`` times keep it, those between
+    are blended linearly by their index; cosines and sines are multiplied by 0.1 ln(factor) + 1."""
+    factor: float
+    original: int
+    fast: float
+    slow: float
+
+
+@dataclass(frozen=True)
+class DovisunAttention:
+    """Grouped-query attention without positions; queries and keys have unit root mean square per head and the
+    softmax's denominator holds one more term exp(0)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+
+
+@dataclass(frozen=True)
+class DovisunLatentAttention:
+    """Attention whose queries and keys/values go through latents; ``rot_dim`` rotated dims shared by all heads."""
+    heads: int
+    dim: int                        # unrotated query / key dims per head
+    rot_dim: int                    # rotated dims per head (the keys' are one vector for all heads)
+    vdim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    rot_base: float
+    rot_scaling: Optional[RotaryScaling]
+
+
+@dataclass(frozen=True)
+class DovisunDense:
+    ff: int
+
+
+@dataclass(frozen=True)
+class DovisunExperts:
+    experts: int
+    top: int
+    ff: int
+
+
+@dataclass(frozen=True)
+class DovisunLayer:
+    type: str                       # "attention" | "latent_attention"
+    mixer: object                   # DovisunAttention | DovisunLatentAttention
+    mlp: object                     # DovisunDense | DovisunExperts | None
+
+
+@dataclass(frozen=True)
+class DovisunConfig:
+    """Keys of a Dovisun config.json: parallel blocks (one RMS norm, a mixer and a feed-forward that both read it)
+    listed layer by layer, a run of layers that is passed several times on the same tensors with the embedding
+    mixed into the stream ahead of every pass (``loop``), a scale on the embedding and a soft cap on the logits."""
+    architecture: str
+    vocab_size: int
+    hidden_size: int
+    layers: tuple                   # of DovisunLayer
+    norm_eps: float
+    embedding_scale: float
+    logit_softcap: float            # 0: none
+    loop_start: int
+    loop_stop: int                  # layers loop_start .. loop_stop - 1 run loop_times times in a row; equal: no loop
+    loop_times: int
+
+    @classmethod
+    def from_dict(cls, d: Mapping[str, Any]) -> "DovisunConfig":
+        norm, emb = d.get("norm") or {}, d.get("embedding") or {}
+        raw_layers = d.get("layers")
+        if not isinstance(raw_layers, (list, tuple)) or not raw_layers:
+            raise ConfigError("config.json: key 'layers' must be a non-empty list")
+        layers = []
+        for i, L in enumerate(raw_layers):
+            try:
+                if not isinstance(L, Mapping):
+                    raise ConfigError("a layer must be an object")
+                kind, m = _take(L, "type", str), L.get("mixer")
+                if not isinstance(m, Mapping):
+                    raise ConfigError("no 'mixer' object")
+                if kind == "attention":
+                    dim = _take(m, "dim", int)
+                    mixer = DovisunAttention(heads=_take(m, "heads", int), kv_heads=_take(m, "kv_heads", int), dim=dim,
+                                             vdim=_take(m, "vdim", int, dim), scale=_take(m, "scale", float))
+                    if mixer.heads < 1 or mixer.kv_heads < 1 or mixer.heads % mixer.kv_heads or dim < 1 or mixer.vdim < 1:
+                        raise ConfigError(f"{mixer.heads} heads over {mixer.kv_heads} kv heads of sizes {dim} and {mixer.vdim}")
+                elif kind == "latent_attention":
+                    rot = m.get("rot") or {}
+                    rot_dim = _take(m, "rot_dim", int)
+                    sc = rot.get("scaling")
+                    scaling = None
+                    if sc is not None:
+                        if not isinstance(sc, Mapping):
+                            raise ConfigError("'rot.scaling' must be an object")
+                        scaling = RotaryScaling(factor=_take(sc, "factor", float), original=_take(sc, "original", int),
+                                                fast=_take(sc, "fast", float), slow=_take(sc, "slow", float))
+                        if scaling.factor <= 0 or scaling.original < 1 or scaling.fast <= 0 or scaling.slow <= 0:
+                            raise ConfigError("'rot.scaling': factor, original, fast and slow must be positive")
+                    dim = _take(m, "dim", int)
+                    mixer = DovisunLatentAttention(
+                        heads=_take(m, "heads", int), dim=dim, rot_dim=rot_dim, vdim=_take(m, "vdim", int, dim),
+                        q_rank=_take(m, "q_rank", int), kv_rank=_take(m, "kv_rank", int), scale=_take(m, "scale", float),
+                        rot_base=_take(rot, "base", float, 10000.0), rot_scaling=scaling)
+                    if _take(rot, "dims", int, rot_dim) != rot_dim:
+                        raise ConfigError(f"'rot.dims' = {rot['dims']} differs from 'rot_dim' = {rot_dim}: the rotated part is rotated whole")
+                    if mixer.heads < 1 or dim < 1 or rot_dim < 0 or rot_dim % 2 or mixer.vdim < 1 \
+                            or mixer.q_rank < 1 or mixer.kv_rank < 1:
+                        raise ConfigError("latent attention sizes must be positive and 'rot_dim' even")
+                else:
+                    raise ConfigError(f"type {kind!r}; known: ['attention', 'latent_attention']")
+                mlp = L.get("mlp")
+                if mlp is not None:
+                    if not isinstance(mlp, Mapping):
+                        raise ConfigError("'mlp' must be null or an object")
+                    mlp_kind = _take(mlp, "kind", str)
+                    if mlp_kind == "dense":
+                        mlp = DovisunDense(ff=_take(mlp, "ff", int))
+                        if mlp.ff < 1:
+                            raise ConfigError("'mlp.ff' must be positive")
+                    elif mlp_kind == "moe":
+                        router, expert = mlp.get("router") or {}, mlp.get("expert") or {}
+                        mlp = DovisunExperts(experts=_take(router, "experts", int), top=_take(router, "top", int),
+                                             ff=_take(expert, "ff", int))
+                        if mlp.ff < 1 or not 1 <= mlp.top <= mlp.experts:
+                            raise ConfigError(f"top = {mlp.top} of {mlp.experts} experts of size {mlp.ff}")
+                    else:
+                        raise ConfigError(f"'mlp.kind' = {mlp_kind!r}; known: ['dense', 'moe']")
+            except ConfigError as e:
+                raise ConfigError(f"{e} (layer {i})") from None
+            layers.append(DovisunLayer(kind, mixer, mlp))
+        loop = d.get("loop") or {}
+        if not isinstance(loop, Mapping):
+            raise ConfigError("config.json: key 'loop' must be an object")
+        start, stop = _take(loop, "start", int, 0), _take(loop, "stop", int, 0)
+        cfg = cls(architecture=_take(d, "architecture", str, "Dovisun"), vocab_size=_take(d, "vocab", int),
+                  hidden_size=_take(d, "width", int), layers=tuple(layers), norm_eps=_take(norm, "eps", float),
+                  embedding_scale=_take(emb, "scale", float, 1.0), logit_softcap=_take(d, "logit_softcap", float, 0.0),
+                  loop_start=start, loop_stop=stop, loop_times=_take(loop, "times", int, 1))
+        if cfg.vocab_size < 1 or cfg.hidden_size < 1 or cfg.norm_eps < 0 or cfg.logit_softcap < 0:
+            raise ConfigError("config.json: 'vocab' and 'width' must be positive, 'norm.eps' and 'logit_softcap' not negative")
+        if not 0 <= start <= stop <= len(layers) or cfg.loop_times < 1:
+            raise ConfigError(f"config.json: 'loop' = layers {start} .. {stop} - 1, {cfg.loop_times} times, of {len(layers)} layers")
+        return cfg
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def loops(self) -> bool:
+        """Whether a run of layers is passed at all (and so the embedding mixed in ahead of each pass)."""
+        return self.loop_stop > self.loop_start

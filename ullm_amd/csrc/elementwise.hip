@@ -377,6 +377,91 @@ extern "C" int ullm_add_bias(void* y, const float* bias, int T_, int N, long lon
   ULLM_LAUNCH_CHECK();
 }
 
+// ------------------------------------------------------------------ activations of an ungated feed-forward
+// out = act(x) element by element on 32-bit values.  ACT_RELU2: max(x, 0)^2.  ACT_GELU_TANH:
+// 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))).
+enum { ACT_RELU2 = 0, ACT_GELU_TANH = 1 };
+__device__ __forceinline__ float activate(float x, int kind) {
+  if (kind == ACT_RELU2) {
+    const float r = fmaxf(x, 0.f);
+    return r * r;
+  }
+  return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+}
+
+template <typename T>
+__global__ void activation_kernel(const T* __restrict__ x, T* __restrict__ out, size_t total, int kind) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  st_f32(out + idx, activate(ld_f32(x + idx), kind));
+}
+
+template <typename T>
+__global__ void activation_vec_kernel(const T* __restrict__ x, T* __restrict__ out, size_t total4, int kind) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total4) return;
+  const float4 v = ld4_f32_stream(x + 4 * idx);
+  st4_f32(out + 4 * idx, make_float4(activate(v.x, kind), activate(v.y, kind), activate(v.z, kind), activate(v.w, kind)));
+}
+
+extern "C" int ullm_activation(const void* x, void* out, long long total, int kind, int dtype, hipStream_t stream) {
+  if (total <= 0) return 0;
+  if (kind != ACT_RELU2 && kind != ACT_GELU_TANH) return ULLM_ERR_UNSUPPORTED;
+  if (total % 4 == 0 && !(((uintptr_t)x | (uintptr_t)out) & 15)) {
+    const size_t total4 = (size_t)total / 4;
+    dim3 vblock(256), vgrid((unsigned)((total4 + 255) / 256));
+    if (dtype == ULLM_F32)
+      hipLaunchKernelGGL(activation_vec_kernel<float>, vgrid, vblock, 0, stream, (const float*)x, (float*)out, total4, kind);
+    else if (dtype == ULLM_BF16)
+      hipLaunchKernelGGL(activation_vec_kernel<bf16_t>, vgrid, vblock, 0, stream, (const bf16_t*)x, (bf16_t*)out, total4, kind);
+    else
+      return ULLM_ERR_DTYPE;
+    ULLM_LAUNCH_CHECK();
+  }
+  dim3 block(256), grid((unsigned)(((size_t)total + 255) / 256));
+  if (dtype == ULLM_F32)
+    hipLaunchKernelGGL(activation_kernel<float>, grid, block, 0, stream, (const float*)x, (float*)out, (size_t)total, kind);
+  else if (dtype == ULLM_BF16)
+    hipLaunchKernelGGL(activation_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)x, (bf16_t*)out, (size_t)total, kind);
+  else
+    return ULLM_ERR_DTYPE;
+  ULLM_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------ the stream beside another 32-bit row
+// residual[t, :] += mult * branch[t, :] (branch may be null), then out[t, :] = [residual[t, :] | other[t, :]] in
+// the compute dtype: the input of a product that mixes the stream with a second stream of the same width.
+template <typename TB, typename TO>
+__global__ void stream_pair_kernel(const TB* __restrict__ branch, float mult, float* __restrict__ residual,
+                                   const float* __restrict__ other, TO* __restrict__ out, int H, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t t = idx / H;
+  const int i = (int)(idx - t * H);
+  float x = residual[idx];
+  if (branch) {
+    x += mult * ld_f32(branch + idx);
+    residual[idx] = x;
+  }
+  st_f32(out + t * (size_t)(2 * H) + i, x);
+  st_f32(out + t * (size_t)(2 * H) + H + i, other[idx]);
+}
+
+extern "C" int ullm_stream_pair(const void* branch, int branch_dtype, float mult, float* residual, const float* other,
+                                void* out, int T_, int H, int dtype, hipStream_t stream) {
+  if (T_ <= 0) return 0;
+  if (H <= 0) return ULLM_ERR_SHAPE;
+  const size_t total = (size_t)T_ * H;
+  dim3 block(256), grid((unsigned)((total + 255) / 256));
+#define GO(TB, TO) hipLaunchKernelGGL((stream_pair_kernel<TB, TO>), grid, block, 0, stream, (const TB*)branch, mult, residual, \
+    other, (TO*)out, H, total)
+  if (dtype == ULLM_F32) { if (branch_dtype == ULLM_BF16) GO(bf16_t, float); else GO(float, float); }
+  else if (dtype == ULLM_BF16) { if (branch_dtype == ULLM_BF16) GO(bf16_t, bf16_t); else GO(float, bf16_t); }
+  else return ULLM_ERR_DTYPE;
+#undef GO
+  ULLM_LAUNCH_CHECK();
+}
+
 // ------------------------------------------------------------------ SiLU(gate) * up
 template <typename T>
 __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
@@ -539,7 +624,8 @@ extern "C" int ullm_sum_stacks(const float* stacks, int n_stacks, const float* b
 
 // ------------------------------------------------------------------ q/k norm + rotary + cache write
 // One wave per (token, head) of the fused projection row  [q heads | k heads | v heads].
-//   q heads: per-head RMS norm (gain shared by all heads, may be null), rotation, written to q_out
+//   q heads: per-head RMS norm (gain shared by all heads, may be null; the mean of squares is taken over norm_dim
+//            values, the head's own size where it is stored padded with zeros), rotation, written to q_out
 //   k heads: the same with the k gain, written into the token's cache page
 //   v heads: copied into the cache page; value head j is head v_head0 + j of the row (nq + nkv where the
 //            row holds values of its own; nq where the values are the keys as projected, before norm and rotation)
@@ -558,7 +644,7 @@ __global__ void qk_norm_rope_write_kernel(
     const float* __restrict__ cos_sin, int table_rows, int rot, int style,
     const int* __restrict__ positions, const int* __restrict__ token_entry,
     const int* __restrict__ block_table, int bt_stride, T* __restrict__ k_pool, T* __restrict__ v_pool,
-    int page_size, int nq, int nkv, int hd, int write_kv, int v_head0) {
+    int page_size, int nq, int nkv, int hd, int write_kv, int v_head0, int norm_dim) {
   __shared__ float vals[MAX_HEAD_DIM];
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int pos = positions[t];
@@ -588,7 +674,7 @@ __global__ void qk_norm_rope_write_kernel(
   }
   if (gain) {
     ss = wave_sum(ss);
-    const float rs = rsqrtf(ss / (float)hd + eps);
+    const float rs = rsqrtf(ss / (float)norm_dim + eps);
     for (int i = lane; i < hd; i += WAVE) vals[i] = (vals[i] * rs) * gain[i];
   }
   __syncthreads();
@@ -685,7 +771,7 @@ qk_norm_rope_write_vec_kernel(
     const int* __restrict__ positions, const int* __restrict__ token_entry,
     const int* __restrict__ block_table, int bt_stride, T* __restrict__ k_pool, T* __restrict__ v_pool,
     int page_size, int nq, int nkv, int hd, int write_kv, int n_tokens, int blocks_per_token, int heads_per_thread,
-    int v_head0) {
+    int v_head0, int norm_dim) {
   if (blockIdx.x >= (unsigned)(n_tokens * blocks_per_token)) {
     value_runs_block<T>(qkv, qkv_stride, positions, token_entry, block_table, bt_stride, v_pool, page_size, v_head0, nkv,
                         hd, n_tokens, (int)blockIdx.x - n_tokens * blocks_per_token);
@@ -744,7 +830,7 @@ qk_norm_rope_write_vec_kernel(
       // pairwise, the most distant lanes of a head first: the decode attention kernel, which does this
       // norm itself for single new tokens, adds in the same order (multiply-adds spelled out in both)
       for (int m = lph >> 1; m > 0; m >>= 1) ss += __shfl_xor(ss, m, WAVE);
-      const float rs = rsqrtf(ss / (float)hd + eps);
+      const float rs = rsqrtf(ss / (float)norm_dim + eps);
       if (arith) {
         const float4 g0 = *reinterpret_cast<const float4*>(gain + d0), g1 = *reinterpret_cast<const float4*>(gain + d0 + 4);
         const float gg[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
@@ -792,9 +878,10 @@ extern "C" int ullm_qk_norm_rope_write(
     const float* k_gain, float eps, const float* cos_sin, int table_rows, int rot, int style,
     const int* positions, const int* token_entry, const int* block_table, int bt_stride,
     void* k_pool, void* v_pool, int page_size, int T_, int nq, int nkv, int hd, int write_kv,
-    int v_head0, int dtype, hipStream_t stream) {
+    int v_head0, int norm_dim, int dtype, hipStream_t stream) {
   if (T_ <= 0) return 0;
   if (hd <= 0 || hd > MAX_HEAD_DIM || nq <= 0 || nkv <= 0 || page_size <= 0) return ULLM_ERR_SHAPE;
+  if (norm_dim <= 0 || norm_dim > hd) return ULLM_ERR_SHAPE;
   if (v_head0 != nq + nkv && v_head0 != nq) return ULLM_ERR_SHAPE;
   if (rot < 0 || rot > hd || (rot & 1) || (style != 0 && style != 1 && style != 2)) return ULLM_ERR_SHAPE;
   if (style != 0 && rot > 0 && (!cos_sin || table_rows <= 0)) return ULLM_ERR_SHAPE;
@@ -825,7 +912,7 @@ extern "C" int ullm_qk_norm_rope_write(
 #define GOV(TT) hipLaunchKernelGGL(qk_norm_rope_write_vec_kernel<TT>, vgrid, vblock, 0, stream, \
     (const TT*)qkv, qkv_stride, (TT*)q_out, q_out_stride, q_gain, k_gain, eps, cos_sin, table_rows, \
     rot, style, positions, token_entry, block_table, bt_stride, (TT*)k_pool, (TT*)v_pool, page_size, \
-    nq, nkv, hd, kv_flags, T_, blocks_per_token, heads_per_thread, v_head0)
+    nq, nkv, hd, kv_flags, T_, blocks_per_token, heads_per_thread, v_head0, norm_dim)
     if (dtype == ULLM_F32) GOV(float);
     else if (dtype == ULLM_BF16) GOV(bf16_t);
     else return ULLM_ERR_DTYPE;
@@ -836,7 +923,7 @@ extern "C" int ullm_qk_norm_rope_write(
 #define GO(TT) hipLaunchKernelGGL(qk_norm_rope_write_kernel<TT>, grid, block, 0, stream, \
     (const TT*)qkv, qkv_stride, (TT*)q_out, q_out_stride, q_gain, k_gain, eps, cos_sin, table_rows, \
     rot, style, positions, token_entry, block_table, bt_stride, (TT*)k_pool, (TT*)v_pool, page_size, \
-    nq, nkv, hd, write_kv, v_head0)
+    nq, nkv, hd, write_kv, v_head0, norm_dim)
   if (dtype == ULLM_F32) GO(float);
   else if (dtype == ULLM_BF16) GO(bf16_t);
   else return ULLM_ERR_DTYPE;

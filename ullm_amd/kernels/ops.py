@@ -209,6 +209,36 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     return out
 
 
+ACT_RELU2, ACT_GELU_TANH = 0, 1       # activations of an ungated feed-forward
+
+
+def activation(x: torch.Tensor, kind: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """act(x) element by element, computed in 32-bit: ACT_RELU2 max(x, 0)^2, ACT_GELU_TANH the tanh form of GELU."""
+    _need(x.is_contiguous(), "activation takes a contiguous tensor")
+    if out is None:
+        out = torch.empty_like(x)
+    _need(out.shape == x.shape and out.is_contiguous() and out.dtype == x.dtype, "bad activation output")
+    _check(build.load("elementwise").ullm_activation(_p(x), _p(out), ctypes.c_longlong(x.numel()), _c_int(kind),
+                                                     _c_int(_dt(x)), _stream()), "activation")
+    return out
+
+
+def stream_pair(branch: Optional[torch.Tensor], mult: float, residual: torch.Tensor, other: torch.Tensor,
+                out_dtype: torch.dtype) -> torch.Tensor:
+    """residual (float32 [T, H], in place) += mult * branch ([T, H] or None); returns [residual | other] as
+    [T, 2 H] of ``out_dtype`` for ``other`` float32 [T, H]."""
+    T, H = residual.shape
+    _need(residual.dtype == torch.float32 and residual.is_contiguous(), "residual must be contiguous float32")
+    _need(other.dtype == torch.float32 and other.is_contiguous() and other.shape == (T, H), "other must be float32 [T, H]")
+    if branch is not None:
+        _need(branch.shape == (T, H) and branch.is_contiguous(), "branch must be contiguous [T, H]")
+    out = torch.empty((T, 2 * H), dtype=out_dtype, device=residual.device)
+    _check(build.load("elementwise").ullm_stream_pair(
+        _p(branch), _c_int(_dt(branch) if branch is not None else F32), _c_float(mult), _p(residual), _p(other), _p(out),
+        _c_int(T), _c_int(H), _c_int(_dt(out)), _stream()), "stream_pair")
+    return out
+
+
 def glu_clamped(gate_up: torch.Tensor, limit: float, alpha: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """g * sigmoid(alpha * g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit), for a contiguous
     [T, 2I] input gate | up."""
@@ -244,12 +274,13 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_out: torch.Tensor, q_gain: Optional[
                        rotary_dim: int, style: int, positions: torch.Tensor, token_entry: torch.Tensor,
                        block_table: torch.Tensor, k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor],
                        page_size: int, nq: int, nkv: int, hd: int, write_kv: bool,
-                       values_from_keys: bool = False) -> None:
+                       values_from_keys: bool = False, norm_dim: int = 0) -> None:
     """Per-head norm and rotation of q (to ``q_out`` [T, nq*hd]) and k, and the cache write of k and v.
     ``qkv`` is [T, (nq + 2 nkv) * hd]; key pool [pages, nkv, page_size, hd], value pool
     [pages, nkv, hd, page_size]; ``block_table`` is
     int32 [B, stride] with one row per batch entry.  With ``values_from_keys`` the row is [T, (nq + nkv) * hd]
-    and the values written are the keys as projected, before norm and rotation."""
+    and the values written are the keys as projected, before norm and rotation.  ``norm_dim``: the size the norm's
+    mean of squares is taken over (heads stored padded with zeros to ``hd``; 0: ``hd``)."""
     T = qkv.shape[0]
     _need(qkv.dim() == 2 and qkv.shape[1] == (nq + (1 if values_from_keys else 2) * nkv) * hd and qkv.stride(1) == 1,
           "bad qkv shape")
@@ -276,7 +307,7 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_out: torch.Tensor, q_gain: Optional[
         _c_float(eps), _p(cos_sin), _c_int(table_rows), _c_int(rotary_dim), _c_int(style), _p(positions),
         _p(token_entry), _p(block_table), _c_int(block_table.stride(0)), _p(k_pool), _p(v_pool),
         _c_int(page_size), _c_int(T), _c_int(nq), _c_int(nkv), _c_int(hd), _c_int(1 if write_kv else 0),
-        _c_int(nq if values_from_keys else nq + nkv), _c_int(_dt(qkv)), _stream()), "qk_norm_rope_write")
+        _c_int(nq if values_from_keys else nq + nkv), _c_int(norm_dim or hd), _c_int(_dt(qkv)), _stream()), "qk_norm_rope_write")
 
 
 
@@ -1053,16 +1084,103 @@ def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
     return out
 
 
+# ---------------------------------------------------------------------------------- latent attention
+
+def latent_prepare(proj: torch.Tensor, q_off: int, q_rank: int, kv_off: int, kv_rank: int, kr_off: int, rot: int,
+                   g_off: int, n_gate: int, q_gain: Optional[torch.Tensor], kv_gain: torch.Tensor, eps: float,
+                   cos_sin: Optional[torch.Tensor], positions: torch.Tensor, token_entry: torch.Tensor,
+                   block_table: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, page_size: int, hd: int,
+                   write_kv: bool, dtype: torch.dtype):
+    """What a latent-attention layer does with its first product ``proj`` (float32 [T, columns]: q latent at ``q_off``,
+    kv latent at ``kv_off``, the rotated key part at ``kr_off``, gate logits at ``g_off``): returns (cq, gate) with
+    cq = rmsnorm(q latent) * ``q_gain`` as [T, q_rank] and gate = the logits as [T, n_gate rounded up to 8], both of
+    ``dtype``; with ``write_kv`` the token's cache row [rmsnorm(kv latent) * ``kv_gain`` | rotated key part] goes to
+    ``k_pool`` ([pages, 1, page_size, hd]) and the normed latent to ``v_pool`` ([pages, 1, hd, page_size])."""
+    T = proj.shape[0]
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1, "proj must be float32 [T, columns]")
+    _i32(positions, "positions", T)
+    _i32(token_entry, "token_entry", T)
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1,
+          "block_table must be int32 [B, stride]")
+    for g, nm, n in ((q_gain, "q_gain", q_rank), (kv_gain, "kv_gain", kv_rank)):
+        _need((g is None and n == 0) or (g is not None and g.dtype == torch.float32 and g.numel() == n and g.is_contiguous()),
+              f"{nm} must be float32 [{n}]")
+    table_rows = 0
+    if rot > 0:
+        _need(cos_sin is not None and cos_sin.dtype == torch.float32 and cos_sin.dim() == 2 and cos_sin.shape[1] == rot
+              and cos_sin.is_contiguous(), "cos_sin must be float32 [positions, rot]")
+        table_rows = cos_sin.shape[0]
+    if write_kv:
+        _check_pools(k_pool, v_pool, 1, page_size, hd, dtype)
+    cq = torch.empty((T, q_rank), dtype=dtype, device=proj.device)
+    ldg = -(-n_gate // 8) * 8
+    gate = torch.zeros((T, ldg), dtype=dtype, device=proj.device) if n_gate else None
+    _check(build.load("latent").ullm_latent_prepare(
+        _p(proj), _c_int(proj.stride(0)), _c_int(q_off), _c_int(q_rank), _c_int(kv_off), _c_int(kv_rank), _c_int(kr_off),
+        _c_int(rot), _c_int(g_off), _c_int(n_gate), _p(q_gain), _p(kv_gain), _c_float(eps), _p(cos_sin), _c_int(table_rows),
+        _p(positions), _p(token_entry), _p(block_table), _c_int(block_table.stride(0)), _p(k_pool), _p(v_pool),
+        _c_int(page_size), _c_int(hd), _c_int(1 if write_kv else 0), _p(cq), _p(gate), _c_int(ldg), _c_int(T),
+        _c_int(F32 if dtype == torch.float32 else BF16), _stream()), "latent_prepare")
+    return cq, gate
+
+
+def head_linear(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y[t, h] = w[h] x[t, h] for x [T, heads, K] (unit stride along K, any strides otherwise), w contiguous
+    [heads, N, K] of x's dtype; y [T, heads, N] (``out`` may be a strided view with unit stride along N).  32-bit sums
+    in an order that depends on the row alone."""
+    T, heads, K = x.shape
+    _need(w.dim() == 3 and w.shape[0] == heads and w.shape[2] == K and w.is_contiguous() and w.dtype == x.dtype,
+          "w must be contiguous [heads, N, K] of x's dtype")
+    _need(x.stride(2) == 1, "x must have unit stride along K")
+    N = w.shape[1]
+    if out is None:
+        out = torch.empty((T, heads, N), dtype=x.dtype, device=x.device)
+    _need(out.shape == (T, heads, N) and out.stride(2) == 1 and out.dtype == x.dtype, "bad head_linear output")
+    ll = ctypes.c_longlong
+    _check(build.load("latent").ullm_head_linear(_p(x), ll(x.stride(0)), ll(x.stride(1)), _p(w), _p(out), ll(out.stride(0)),
+                                                 ll(out.stride(1)), _c_int(T), _c_int(heads), _c_int(N), _c_int(K),
+                                                 _c_int(_dt(x)), _stream()), "head_linear")
+    return out
+
+
+def latent_query(qa: torch.Tensor, q: torch.Tensor, plain: int, rot: int, hd: int, cos_sin: Optional[torch.Tensor],
+                 positions: torch.Tensor) -> torch.Tensor:
+    """The query rows [T, heads * hd] a latent-attention layer hands the attention kernels: per head
+    [qa[t, h] (rank values) | the head's last ``rot`` dims of ``q`` turned by the token's position | zeros], for
+    qa [T, heads, rank] (unit stride along rank) and q [T, heads * (plain + rot)]."""
+    T, heads, rank = qa.shape
+    _need(qa.stride(2) == 1 and q.dtype == qa.dtype and q.dim() == 2 and q.stride(1) == 1
+          and q.shape == (T, heads * (plain + rot)), "qa must be [T, heads, rank], q [T, heads * (plain + rot)]")
+    _i32(positions, "positions", T)
+    table_rows = 0
+    if rot > 0:
+        _need(cos_sin is not None and cos_sin.dtype == torch.float32 and cos_sin.dim() == 2 and cos_sin.shape[1] == rot
+              and cos_sin.is_contiguous(), "cos_sin must be float32 [positions, rot]")
+        table_rows = cos_sin.shape[0]
+    out = torch.empty((T, heads * hd), dtype=qa.dtype, device=qa.device)
+    ll = ctypes.c_longlong
+    _check(build.load("latent").ullm_latent_query(_p(qa), ll(qa.stride(0)), ll(qa.stride(1)), _p(q), _c_int(q.stride(0)),
+                                                  _c_int(plain), _c_int(rot), _c_int(rank), _c_int(heads), _c_int(hd),
+                                                  _p(cos_sin), _c_int(table_rows), _p(positions), _p(out),
+                                                  _c_int(out.stride(0)), _c_int(T), _c_int(_dt(qa)), _stream()),
+           "latent_query")
+    return out
+
+
 # ---------------------------------------------------------------------------------- routed feed-forward
 
 MOE_MAX_ROUTER, MOE_MAX_TOP = 1024, 32
 MOE_TILE_ROWS = (16, 32, 64, 128)     # grouped rows a block of the matrix-core expert products takes
 
 
-def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int):
+ROUTE_SOFTMAX_ALL, ROUTE_TOP_LOGITS = 0, 1      # how a router turns logits into experts and weights
+
+
+def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, mode: int = ROUTE_SOFTMAX_ALL):
     """(ids int32 [T, top], weights float32 [T, top]) from router logits float32 [T, R]: the softmax over all R, the
     ``top`` largest of softmax + ``correction`` (float32 [R] or None; ties go to the lower index), and as weights the
-    chosen outputs' softmax values over their sum (+ 1e-20)."""
+    chosen outputs' softmax values over their sum (+ 1e-20).  With ``mode`` ROUTE_TOP_LOGITS: the ``top`` largest of
+    logits + ``correction`` (a bias on the logits), weighed by the softmax over those alone."""
     T, R = logits.shape
     _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "router logits must be float32 [T, R]")
     _need(1 <= top <= min(R, MOE_MAX_TOP) and R <= MOE_MAX_ROUTER, f"top {top} of {R} router outputs: at most "
@@ -1073,14 +1191,15 @@ def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int
     ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
     _check(build.load("moe").ullm_moe_route(_p(logits), _c_int(logits.stride(0)), _p(correction), _c_int(T), _c_int(R),
-                                            _c_int(top), _p(ids), _p(weights), _stream()), "moe_route")
+                                            _c_int(top), _p(ids), _p(weights), _c_int(mode), _stream()), "moe_route")
     return ids, weights
 
 
 MOE_ROUTER_MAX_WIDTH = 12288      # widest row the fused router kernel keeps in shared memory
 
 
-def moe_router(x: torch.Tensor, w_router: torch.Tensor, correction: Optional[torch.Tensor], top: int):
+def moe_router(x: torch.Tensor, w_router: torch.Tensor, correction: Optional[torch.Tensor], top: int,
+               mode: int = ROUTE_SOFTMAX_ALL):
     """:func:`moe_route` of the 32-bit product of ``x`` [T, H] with ``w_router`` (float32 [R, H]), in one kernel: every
     router output is summed along the row in an order that depends on nothing but the row."""
     T, H = x.shape
@@ -1096,8 +1215,8 @@ def moe_router(x: torch.Tensor, w_router: torch.Tensor, correction: Optional[tor
     ids = torch.empty((T, top), dtype=torch.int32, device=x.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=x.device)
     _check(build.load("moe").ullm_moe_router(_p(x), _c_int(x.stride(0)), _p(w_router), _p(correction), _c_int(T), _c_int(H),
-                                             _c_int(R), _c_int(top), _p(ids), _p(weights), _c_int(_dt(x)), _stream()),
-           "moe_router")
+                                             _c_int(R), _c_int(top), _p(ids), _p(weights), _c_int(mode), _c_int(_dt(x)),
+                                             _stream()), "moe_router")
     return ids, weights
 
 

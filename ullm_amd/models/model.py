@@ -73,6 +73,7 @@ class Model:
             if not (0 <= layer < len(self.blocks)):
                 raise ValueError(f"run order names layer {layer}: out of range")
             self.cache_owner.setdefault(cache_id, idx)
+        self._keeps_embedding = any(b.needs_embedding for b in self.blocks)
         self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
         self.head_bias: Optional[torch.Tensor] = None
@@ -159,6 +160,8 @@ class Model:
         else:
             residual = ops.embedding(ctx.token_ids, self.embedding, scale=self.plan.embedding_scale)
         pending = None
+        if self._keeps_embedding:
+            ctx.embedded = residual.clone()      # the stream's rows are written in place from here on
         for idx, (layer, cache_id) in enumerate(self.run_order):
             cache = caches.get(cache_id)
             if cache is None:

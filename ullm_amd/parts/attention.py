@@ -12,7 +12,9 @@ query/key size (``value_dim``), the q/k norm taken over the whole projection ins
 with ``score_bias()``), a gate per head on the heads' outputs (``head_gate``: sigmoid of one more projection of
 the mixer's input), no key/value projections of its own (``own_kv=False``: the layer reads the cache another
 layer writes), values that are the keys as projected, before rotation (``values="keys"``: no value projection),
-a sink per head in the softmax's denominator (``sink``: a learned number with no key and no value), biases on the
+a sink per head in the softmax's denominator (``sink``: a learned number with no key and no value; ``sink_value``:
+the same number for every head, a constant of the design without a tensor), a per-head norm without gains
+(``qk_norm_gain=False``: queries and keys are only divided by their root mean square), biases on the
 projections also there (``bias`` on q, k and v, ``out_bias`` on the output) and other tensor names (``names``).
 Any of these takes the general path below: one projection
 q | k | v | gate, heads padded with zeros to a size the attention kernels take (zero key dims add nothing to a
@@ -93,7 +95,8 @@ class GQAttention(Mixer):
                  bias: bool = False, window: int = 0, scale: Optional[float] = None,
                  value_dim: Optional[int] = None, qk_norm: str = "head", head_gate: bool = False,
                  own_kv: bool = True, names: Optional[Dict[str, str]] = None, values: str = "own",
-                 sink: bool = False, out_bias: bool = False):
+                 sink: bool = False, out_bias: bool = False, sink_value: Optional[float] = None,
+                 qk_norm_gain: bool = True):
         if qk_norm not in ("head", "whole"):
             raise ValueError(f"qk_norm={qk_norm!r}: 'head' (per head) or 'whole' (over the whole projection)")
         if values not in ("own", "keys"):
@@ -101,18 +104,22 @@ class GQAttention(Mixer):
         self.dim, self.vdim = head_dim, head_dim if value_dim is None else int(value_dim)
         self.qk_norm, self.head_gate, self.own_kv = qk_norm, bool(head_gate), bool(own_kv)
         self.values_are_keys, self.sink, self.out_bias = values == "keys", bool(sink), bool(out_bias)
+        self.sink_value = None if sink_value is None else float(sink_value)
+        self.norm_has_gain = bool(qk_norm_gain)
+        if self.sink and self.sink_value is not None:
+            raise ValueError("a sink is a learned tensor (sink) or one constant (sink_value), not both")
+        if not self.norm_has_gain and (qk_norm != "head" or qk_norm_eps is None):
+            raise ValueError("a norm without gains is the per-head norm (qk_norm='head' with an eps)")
         self.names = {**DEFAULT_NAMES, **(names or {})}
         self.general = (self.vdim != head_dim or qk_norm == "whole" or self.head_gate or not self.own_kv
                         or names is not None or self.values_are_keys or self.sink or self.out_bias
+                        or self.sink_value is not None or not self.norm_has_gain
                         or (position is not None and type(position).score_bias is not PositionEncoding.score_bias))
         if self.general:
             if self.values_are_keys and (self.vdim != head_dim or qk_norm == "whole" or not self.own_kv):
                 raise ValueError("values that are the keys need keys of the layer's own, of the values' size, "
                                  "and no norm over the whole projection")
-            padded = padded_head_size(head_dim, self.vdim)
-            if qk_norm == "head" and qk_norm_eps is not None and padded != head_dim:
-                raise ValueError(f"a per-head norm over heads of {head_dim} stored as {padded}: not built")
-            head_dim = padded
+            head_dim = padded_head_size(head_dim, self.vdim)
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} kv heads")
         if head_dim % 2 or head_dim > 512:
@@ -227,7 +234,7 @@ class GQAttention(Mixer):
             out.append(WeightDecl(self._name("o_bias"), (H,), keep_fp32=True))
         if self.sink:
             out.append(WeightDecl(self._name("sink"), (nq,), keep_fp32=True))
-        if self.qk_norm_eps is not None:
+        if self.qk_norm_eps is not None and self.norm_has_gain:
             per = d if self.qk_norm == "head" else None
             out.append(WeightDecl(self._name("q_norm"), (per or nq * d,), init="gain", keep_fp32=True))
             if self.own_kv:
@@ -269,8 +276,9 @@ class GQAttention(Mixer):
         self.w_qkv = torch.cat(pieces, dim=0).contiguous()
         self.b_qkv = torch.cat(biases, dim=0).contiguous() if self.bias else None
         self.b_o = tensors[self._name("o_bias")].contiguous() if self.out_bias else None
-        if self.sink:
-            self.sinks = tensors[self._name("sink")].to(torch.float32).contiguous()
+        if self.sink or self.sink_value is not None:
+            self.sinks = (tensors[self._name("sink")].to(torch.float32).contiguous() if self.sink else
+                          torch.full((nq,), self.sink_value, dtype=torch.float32, device=env.device))
             self.sinks_log2 = (self.sinks * math.log2(math.e)).contiguous()
         w_o = tensors[self._name("o")]
         if dv != hd:
@@ -280,8 +288,13 @@ class GQAttention(Mixer):
         self.w_o = w_o.contiguous()
         if self.qk_norm_eps is not None:
             if self.qk_norm == "head":
-                self.q_gain = tensors[self._name("q_norm")].contiguous()
-                self.k_gain = tensors[self._name("k_norm")].contiguous() if self.own_kv else None
+                # a head's gains, padded like the head (the padded values are zeros whatever they are multiplied by)
+                def head_gain(role):
+                    g = (tensors[self._name(role)].to(torch.float32) if self.norm_has_gain
+                         else torch.ones((d,), dtype=torch.float32, device=env.device))
+                    return torch.cat((g, g.new_ones((hd - d,)))).contiguous()
+                self.q_gain = head_gain("q_norm")
+                self.k_gain = head_gain("k_norm") if self.own_kv else None
             else:
                 self.q_gain = heads_padded(tensors[self._name("q_norm")], nq, d).contiguous()
                 self.k_gain = heads_padded(tensors[self._name("k_norm")], nkv, d).contiguous() if self.own_kv else None
@@ -301,7 +314,7 @@ class GQAttention(Mixer):
             ops.qk_norm_rope_write(proj[:, :(nq + kv_heads) * hd], q, self.q_gain, self.k_gain, self.qk_norm_eps or 0.0,
                                    table, rot, style, ctx.positions, ctx.token_entry, group.block_table, cache.k_pool,
                                    cache.v_pool, group.page_size, nq, nkv, hd, write_kv=True,
-                                   values_from_keys=self.values_are_keys)
+                                   values_from_keys=self.values_are_keys, norm_dim=self.dim)
         else:
             if style != 0 and rot > 0 or (self.qk_norm == "head" and self.qk_norm_eps is not None):
                 raise NotImplementedError("rotation or a per-head norm without keys of the layer's own: not built")

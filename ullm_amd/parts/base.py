@@ -201,6 +201,9 @@ class StepContext:
     # every norm of the model takes a stack [S, T, hidden] of float32 partial sums as its branch and
     # adds them up (Norm.adds_stacks): a mixer or feed-forward may then return such a stack
     stacked_branches: bool = False
+    # the embedding output (float32 [T, hidden], never written again), kept by the model where one of its blocks
+    # says ``needs_embedding``; None otherwise
+    embedded: Optional[torch.Tensor] = None
 
 
 # --------------------------------------------------------------------------- parts
@@ -376,6 +379,7 @@ class Block(Part):
     which is only ever given to the block whose ``entry_norm()`` it is."""
     kind = "block"
     hands_norm_ahead = False
+    needs_embedding = False          # the block reads ``ctx.embedded``, the embedding output of the step
 
     def entry_norm(self) -> Optional["Norm"]:
         return None

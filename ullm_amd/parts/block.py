@@ -145,3 +145,43 @@ class ParallelBlock(Block):
         ops.residual_add(mixed, total)
         ops.residual_add(_one_branch(self.ffn.forward(h, ctx)), total)
         return residual, NormedBranch(total, None, self.mult)
+
+
+@register_part("block", "mix_in_embedding")
+class MixInEmbedding(Block):
+    """Not a layer of sublayers but a step between layers: the stream is replaced by a product of itself and the
+    embedding output side by side, x <- W [x ; e] with W [hidden, 2 hidden] (the stream's columns first).  A model
+    that passes a run of layers several times puts it ahead of every pass.  It keeps nothing between steps.  The
+    model hands every block the embedding output as ``ctx.embedded`` if one of its blocks says ``needs_embedding``.
+    What is pending joins the stream in the kernel that lays the two rows side by side; the product's 32-bit
+    sums are the new stream."""
+    needs_embedding = True
+
+    def __init__(self, hidden_size: int, weight_name: str):
+        self.hidden_size, self.weight_name = int(hidden_size), weight_name
+        self.w: Optional[torch.Tensor] = None
+
+    def weights(self):
+        from .base import WeightDecl
+        return [WeightDecl(self.weight_name, (self.hidden_size, 2 * self.hidden_size))]
+
+    def bind(self, tensors, env) -> None:
+        self.w = tensors[self.weight_name].contiguous()
+
+    def forward(self, residual, pending, ctx: StepContext, cache: LayerCache):
+        from .linear import linear
+        if ctx.embedded is None:
+            raise RuntimeError("mix_in_embedding: the model did not keep the embedding output")
+        branch, mult = None, 1.0
+        if isinstance(pending, NormedBranch):
+            if pending.post is not None:
+                # a norm stands behind the branch: the general add kernel applies it; no norm of the stream is asked for
+                ops.add_norm_general(pending.branch, residual, None, 0.0, ops.NORM_RMS, None,
+                                     post_gain=pending.post.kernel_form()[0], post_eps=pending.post.kernel_form()[1],
+                                     post_kind=pending.post.kernel_form()[2], mult=pending.mult)
+            else:
+                branch, mult = _one_branch(pending.branch), pending.mult
+        elif pending is not None and not isinstance(pending, PendingNorm):
+            branch = _one_branch(pending)
+        both = ops.stream_pair(branch, mult, residual, ctx.embedded, ctx.dtype)
+        return linear(both, self.w, out_dtype=torch.float32), None

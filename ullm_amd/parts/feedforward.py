@@ -10,7 +10,7 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, PartEnv, StepContext, WeightDecl, register_part
-from .linear import add_into_stream, can_fuse, gate_up, linear_into_stream, linear_of_norm
+from .linear import add_into_stream, can_fuse, gate_up, linear, linear_into_stream, linear_of_norm
 
 
 @register_part("ffn", "swiglu")
@@ -47,3 +47,33 @@ class SwiGLU(FeedForward):
     def forward_fused(self, x, residual, ctx: StepContext, then=None):
         act = linear_of_norm(x, self.w_gate_up, silu=True)     # the norm before, silu(gate) * up behind the first product
         return add_into_stream(act, self.w_down, residual, then, ctx.dtype)   # residual add (and the next norm's part) behind the second
+
+
+ACTIVATIONS = {"relu2": ops.ACT_RELU2, "gelu_tanh": ops.ACT_GELU_TANH}
+
+
+@register_part("ffn", "mlp")
+class MLP(FeedForward):
+    """Dense feed-forward without a gate: down(act(up(x))), no biases; ``activation`` is "relu2" (the square of
+    relu) or "gelu_tanh".  The activation is applied to the product as stored (bfloat16 or float32) in 32-bit."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, prefix: str, activation: str = "relu2",
+                 names: Optional[Dict[str, str]] = None):
+        if activation not in ACTIVATIONS:
+            raise ValueError(f"activation={activation!r}; known: {sorted(ACTIVATIONS)}")
+        self.hidden_size, self.intermediate_size, self.prefix = hidden_size, intermediate_size, prefix
+        self.act = ACTIVATIONS[activation]
+        self.names = {"up": "up_proj.weight", "down": "down_proj.weight", **(names or {})}
+        self.w_up = self.w_down = None
+
+    def weights(self) -> List[WeightDecl]:
+        p, H, I, n = self.prefix, self.hidden_size, self.intermediate_size, self.names
+        return [WeightDecl(f"{p}.{n['up']}", (I, H)), WeightDecl(f"{p}.{n['down']}", (H, I))]
+
+    def bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
+        self.w_up = tensors[f"{self.prefix}.{self.names['up']}"].contiguous()
+        self.w_down = tensors[f"{self.prefix}.{self.names['down']}"].contiguous()
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        up = linear(x, self.w_up)
+        return linear_into_stream(ops.activation(up, self.act, out=up), self.w_down, ctx)

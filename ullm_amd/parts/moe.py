@@ -7,6 +7,9 @@ output (``correction``), the weights by the chosen outputs' scores alone, divide
 ``down(act(gate(x), up(x)))`` without biases, with the clamped gated unit
 ``act(g, u) = g' * sigmoid(alpha * g') * (u' + 1)``, ``g' = min(g, limit)``, ``u' = clamp(u, -limit, limit)``.
 A shared expert of the same form (sizes and limit of its own) may run for every token and is added.
+Two more forms, each a parameter: ``routing="top_logits"`` picks the ``top`` largest of logits + a learned bias per
+output (the ``correction`` tensor, then a bias on the logits) and weighs them by the softmax over the picked ones
+alone; ``limit=None`` makes every expert the plain gated unit ``silu(g) * u``.
 
 The experts' matrices are stacked ([experts, 2 ff, hidden] with gate rows, then up rows, per expert, and
 [experts, hidden, ff]); the loader puts the checkpoint's per-expert tensors into their rows.  A step groups
@@ -42,9 +45,14 @@ def tile_rows_for(tokens: int, top: int, experts: int) -> int:
 
 @register_part("ffn", "routed_experts")
 class RoutedExperts(FeedForward):
-    def __init__(self, hidden_size: int, experts: int, intermediate_size: int, top: int, limit: float, prefix: str,
-                 identity: int = 0, alpha: float = 1.702, correction: bool = True,
-                 shared_size: int = 0, shared_limit: Optional[float] = None, names: Optional[Dict[str, str]] = None):
+    def __init__(self, hidden_size: int, experts: int, intermediate_size: int, top: int, limit: Optional[float],
+                 prefix: str, identity: int = 0, alpha: float = 1.702, correction: bool = True,
+                 shared_size: int = 0, shared_limit: Optional[float] = None, names: Optional[Dict[str, str]] = None,
+                 routing: str = "softmax_all"):
+        if routing not in ("softmax_all", "top_logits"):
+            raise ValueError(f"routing={routing!r}: 'softmax_all' or 'top_logits'")
+        self.mode = ops.ROUTE_TOP_LOGITS if routing == "top_logits" else ops.ROUTE_SOFTMAX_ALL
+        limit = 0.0 if limit is None else limit            # the kernels read a limit of 0 as the plain unit
         if experts < 0 or identity < 0 or experts + identity < 1:
             raise ValueError(f"{experts} experts and {identity} identity experts: a router needs at least one output")
         if not 1 <= top <= experts + identity:
@@ -98,9 +106,9 @@ class RoutedExperts(FeedForward):
     def route(self, x: torch.Tensor):
         """(ids int32 [T, top], weights float32 [T, top]) of the rows of x."""
         if self.hidden_size <= ops.MOE_ROUTER_MAX_WIDTH:
-            return ops.moe_router(x, self.w_router, self.correction, self.top)     # the product and the routing in one
+            return ops.moe_router(x, self.w_router, self.correction, self.top, self.mode)     # the product and the routing in one
         logits = ops.gemm_simple(x, self.w_router, out_dtype=torch.float32)       # 32-bit sums in a fixed order
-        return ops.moe_route(logits, self.correction, self.top)
+        return ops.moe_route(logits, self.correction, self.top, self.mode)
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         return self.forward_onto(x, ctx, None, None)

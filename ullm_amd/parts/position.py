@@ -26,10 +26,16 @@ class NoPosition(PositionEncoding):
 
 @register_part("position", "rotary")
 class Rotary(PositionEncoding):
-    """``rotary_dim`` leading dims of each head are rotated; ``pairing`` is "half" or "adjacent"."""
+    """``rotary_dim`` leading dims of each head are rotated; ``pairing`` is "half" or "adjacent".
+
+    ``scaling`` = (factor, original, fast, slow) stretches the frequencies by wavelength: with
+    d(t) = rotary_dim * ln(original / (2 pi t)) / (2 ln theta), the pair index at which a pair turns t times over
+    ``original`` positions, lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)), rotary_dim - 1) and
+    ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns at f_i / factor * ramp_i + f_i * (1 - ramp_i),
+    and every cosine and sine is multiplied by 0.1 ln(factor) + 1."""
 
     def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None,
-                 pairing: str = "half", max_positions: Optional[int] = None):
+                 pairing: str = "half", max_positions: Optional[int] = None, scaling: Optional[tuple] = None):
         self.head_dim = head_dim
         self.theta = float(theta)
         self.rotary_dim = head_dim if rotary_dim is None else rotary_dim
@@ -39,19 +45,37 @@ class Rotary(PositionEncoding):
             raise ValueError(f"unknown rotary pairing {pairing!r}")
         self.style = 1 if pairing == "half" else 2
         self.max_positions = max_positions
+        self.scaling = None if scaling is None else tuple(float(v) for v in scaling)
+        if self.scaling is not None and (len(self.scaling) != 4 or min(self.scaling) <= 0):
+            raise ValueError(f"scaling={scaling!r}: (factor, original, fast, slow), all positive")
         self.table: Optional[torch.Tensor] = None
 
     @staticmethod
-    def make_table(rotary_dim: int, theta: float, rows: int) -> torch.Tensor:
-        inv_freq = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
-        angles = torch.arange(rows, dtype=torch.float32)[:, None] * inv_freq[None, :]
-        return torch.cat((angles.cos(), angles.sin()), dim=-1).contiguous()
+    def make_table(rotary_dim: int, theta: float, rows: int, scaling: Optional[tuple] = None) -> torch.Tensor:
+        if scaling is None:
+            inv_freq = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
+            angles = torch.arange(rows, dtype=torch.float32)[:, None] * inv_freq[None, :]
+            return torch.cat((angles.cos(), angles.sin()), dim=-1).contiguous()
+        # stretched frequencies: built in 64-bit, so that the 32-bit table is the rounding of the exact angles' values
+        factor, original, fast, slow = scaling
+        i = torch.arange(rotary_dim // 2, dtype=torch.float64)
+        inv_freq = torch.pow(torch.tensor(float(theta), dtype=torch.float64), -2.0 * i / rotary_dim)
+
+        def pair_turning(times: float) -> float:
+            return rotary_dim * math.log(original / (2 * math.pi * times)) / (2 * math.log(theta))
+        lo = max(math.floor(pair_turning(fast)), 0)
+        hi = min(math.ceil(pair_turning(slow)), rotary_dim - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        inv_freq = inv_freq / factor * ramp + inv_freq * (1.0 - ramp)
+        magnitude = 0.1 * math.log(factor) + 1.0
+        angles = torch.arange(rows, dtype=torch.float64)[:, None] * inv_freq[None, :]
+        return (torch.cat((angles.cos(), angles.sin()), dim=-1) * magnitude).to(torch.float32).contiguous()
 
     def bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
         rows = env.context_len if self.max_positions is None else min(env.context_len, self.max_positions)
         # every layer with the same rotation shares one table: built once, read by all their kernels
-        self.table = env.shared(("rotary", self.rotary_dim, self.theta, rows),
-                                lambda: self.make_table(self.rotary_dim, self.theta, rows).to(env.device))
+        self.table = env.shared(("rotary", self.rotary_dim, self.theta, rows, self.scaling),
+                                lambda: self.make_table(self.rotary_dim, self.theta, rows, self.scaling).to(env.device))
 
     def kernel_args(self):
         return self.table, self.rotary_dim, self.style

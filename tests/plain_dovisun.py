@@ -171,3 +171,56 @@ def forward(w, cfg: dict, tokens, streams: Optional[list] = None) -> torch.Tenso
     z = (rms(x, cfg["norm"]["eps"]) * w["final.norm"]) @ w["head"].T
     cap = cfg.get("logit_softcap") or 0.0
     return cap * torch.tanh(z / cap) if cap > 0 else z
+
+
+def greedy_generate(w, cfg, prompt: List[int], n: int) -> List[int]:
+    toks, out = list(prompt), []
+    for _ in range(n):
+        nxt = int(forward(w, cfg, toks)[-1].argmax())
+        toks.append(nxt)
+        out.append(nxt)
+    return out
+
+
+def random_weights(cfg: dict, seed: int, std: float = 0.08, router_bias_std: float = 0.3):
+    """bfloat16 tensors under the design's names.  The router's logits are about a unit and a half wide whatever
+    the width and its biases a third of a unit, so that a bias left out or added to the weights moves the choice;
+    the mixing matrix ahead of a pass keeps the stream's size."""
+    g = torch.Generator().manual_seed(seed)
+    H = cfg["width"]
+
+    def mat(*shape, s=std):
+        return (torch.randn(*shape, generator=g) * s).bfloat16()
+
+    def gain(n):
+        return (1 + 0.2 * torch.randn(n, generator=g)).bfloat16()
+
+    w = {"embed": mat(cfg["vocab"], H, s=0.5), "head": mat(cfg["vocab"], H, s=0.3), "final.norm": gain(H)}
+    if cfg.get("loop"):
+        w["loop.in"] = mat(H, 2 * H, s=0.7 / math.sqrt(H))
+    for i, L in enumerate(cfg["layers"]):
+        p, m = f"l{i}", L["mixer"]
+        w[f"{p}.norm1"] = gain(H)
+        if L["type"] == "attention":
+            w[f"{p}.mix.q"], w[f"{p}.mix.k"] = mat(m["heads"] * m["dim"], H, s=0.25), mat(m["kv_heads"] * m["dim"], H, s=0.25)
+            w[f"{p}.mix.v"], w[f"{p}.mix.o"] = mat(m["kv_heads"] * m["vdim"], H, s=0.25), mat(H, m["heads"] * m["vdim"])
+        else:
+            d, r = m["dim"], m["rot_dim"]
+            w[f"{p}.mix.dq"], w[f"{p}.mix.dq.norm"] = mat(m["q_rank"], H, s=0.25), gain(m["q_rank"])
+            w[f"{p}.mix.uq"] = mat(m["heads"] * (d + r), m["q_rank"], s=0.25)
+            w[f"{p}.mix.dkv"], w[f"{p}.mix.dkv.norm"] = mat(m["kv_rank"] + r, H, s=0.25), gain(m["kv_rank"])
+            w[f"{p}.mix.uk"], w[f"{p}.mix.uv"] = mat(m["heads"] * d, m["kv_rank"], s=0.25), mat(m["heads"] * m["vdim"], m["kv_rank"], s=0.2)
+            w[f"{p}.mix.g"], w[f"{p}.mix.o"] = mat(m["heads"], H, s=0.3), mat(H, m["heads"] * m["vdim"])
+        f = L.get("mlp")
+        if f is None:
+            continue
+        if f["kind"] == "dense":
+            w[f"{p}.mlp.up"], w[f"{p}.mlp.down"] = mat(f["ff"], H, s=0.25), mat(H, f["ff"])
+            continue
+        n = f["router"]["experts"]
+        w[f"{p}.mlp.router"], w[f"{p}.mlp.router.b"] = mat(n, H, s=1.5 / math.sqrt(H)), mat(n, s=router_bias_std)
+        for e in range(n):
+            ff = f["expert"]["ff"]
+            w[f"{p}.mlp.e{e}.gate"], w[f"{p}.mlp.e{e}.up"] = mat(ff, H, s=0.3), mat(ff, H, s=0.3)
+            w[f"{p}.mlp.e{e}.down"] = mat(H, ff)
+    return w

@@ -489,6 +489,7 @@ class DovisunConfig:
     loop_start: int
     loop_stop: int                  # layers loop_start .. loop_stop - 1 run loop_times times in a row; equal: no loop
     loop_times: int
+    has_loop: bool = False          # config.json has a 'loop' object (and so the checkpoint the mixing matrix)
 
     @classmethod
     def from_dict(cls, d: Mapping[str, Any]) -> "DovisunConfig":
@@ -561,7 +562,8 @@ class DovisunConfig:
         cfg = cls(architecture=_take(d, "architecture", str, "Dovisun"), vocab_size=_take(d, "vocab", int),
                   hidden_size=_take(d, "width", int), layers=tuple(layers), norm_eps=_take(norm, "eps", float),
                   embedding_scale=_take(emb, "scale", float, 1.0), logit_softcap=_take(d, "logit_softcap", float, 0.0),
-                  loop_start=start, loop_stop=stop, loop_times=_take(loop, "times", int, 1))
+                  loop_start=start, loop_stop=stop, loop_times=_take(loop, "times", int, 1),
+                  has_loop=d.get("loop") is not None)
         if cfg.vocab_size < 1 or cfg.hidden_size < 1 or cfg.norm_eps < 0 or cfg.logit_softcap < 0:
             raise ConfigError("config.json: 'vocab' and 'width' must be positive, 'norm.eps' and 'logit_softcap' not negative")
         if not 0 <= start <= stop <= len(layers) or cfg.loop_times < 1:

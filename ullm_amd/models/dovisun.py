@@ -50,10 +50,12 @@ def dovisun_plan(cfg: DovisunConfig) -> ModelPlan:
                 routing="top_logits", correction=True, names={"correction": "router.b"}))
         layers.append(Choice("block", "parallel", params))
     n = len(layers)
-    if cfg.loops:
-        # one more "layer": the step ahead of every pass; its entries in the run order keep nothing, the passes'
-        # layers get cache ids of their own (the first pass the layers' own numbers, later passes numbers behind them)
+    if cfg.has_loop or cfg.loops:
+        # one more "layer": the step ahead of every pass (declared with the tensor also where no layer is passed)
         layers.append(Choice("block", "mix_in_embedding", dict(hidden_size=H, weight_name="loop.in")))
+    if cfg.loops:
+        # its entries in the run order keep nothing; the passes' layers get cache ids of their own (the first pass
+        # the layers' own numbers, later passes numbers behind them)
         order, next_id = [(i, i) for i in range(cfg.loop_start)], n + 1
         for turn in range(cfg.loop_times):
             order.append((n, next_id))

@@ -64,6 +64,8 @@ def dovisun_plan(cfg: DovisunConfig) -> ModelPlan:
                 order.append((i, i) if turn == 0 else (i, next_id))
                 next_id += turn > 0
         order += [(i, i) for i in range(cfg.loop_stop, n)]
+    elif cfg.has_loop:
+        order = [(i, i) for i in range(n)]       # the declared step is never run
     else:
         order = None
     return ModelPlan(

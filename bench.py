@@ -55,9 +55,11 @@ def parse_args():
                     help="instead of the default workload: Pamopel (attention with a distance bias and head gates, a "
                          "layer on another's keys and values, a Mamba-2 layer) beside a Qwen3 stack of the same width, "
                          f"heads, feed-forward, vocabulary and depth, random weights; shapes: {sorted(DESIGN_SHAPES)}")
-    ap.add_argument("--design-model", choices=("both", "all", "pamopel", "qwen3", "ziferax"), default="both",
-                    help="with --design: one design only (for profiles), Pamopel and Qwen3 (both), or these and Ziferax "
-                         "(all: a stack of parallel blocks of windowed attention with sinks and a routed feed-forward)")
+    ap.add_argument("--design-model", choices=("both", "all", "pamopel", "qwen3", "ziferax", "dovisun"), default="both",
+                    help="with --design: one design only (for profiles), Pamopel and Qwen3 (both), or these, Ziferax "
+                         "(a stack of parallel blocks of windowed attention with sinks and a routed feed-forward) and "
+                         "Dovisun (parallel blocks of unit-norm attention with a fixed sink or latent attention, dense "
+                         "or routed feed-forwards, two layers passed twice) (all)")
     ap.add_argument("--prefill-only", type=int, default=0, metavar="T",
                     help="only time a T-token prompt and print its figures (for profiling)")
     return ap.parse_args()
@@ -167,20 +169,44 @@ def ziferax_config(shape):
                 layers=[dict(type="attention", mixer=mixer, mlp=mlp) for _ in range(L)])
 
 
+# Dovisun at a design shape: the same width and heads; six layers of which the third and fourth are passed twice, so
+# eight layer runs a token as the other stacks have; attention layers without positions (unit-norm queries and keys, a
+# fixed sink) and one latent-attention layer in four (a kv latent of 192 and 64 rotated dims: 256 cached values a
+# token, the largest head the matrix-core attention kernels take, against 2 * 8 * 128 of an attention layer; a q
+# latent of 3/8 of the width); dense feed-forwards of the dense
+# stack's size without a gate, and routed ones of as many columns a token (top 4 of 32 experts of a sixth of it).
+def dovisun_config(shape):
+    (W, H, G, D, F, L), _ = DESIGN_SHAPES[shape]
+    att = dict(heads=H, kv_heads=G, dim=D, vdim=D, scale=D ** -0.5)
+    latent = dict(heads=H, dim=D, rot_dim=D // 2, vdim=D, q_rank=W * 3 // 8, kv_rank=192, scale=(D + D // 2) ** -0.5,
+                  rot=dict(base=1e6, dims=D // 2, scaling=dict(factor=8.0, original=4096, fast=32.0, slow=1.0)))
+    dense = dict(kind="dense", ff=F)
+    moe = dict(kind="moe", router=dict(experts=32, top=4), expert=dict(ff=F // 6))
+    layers = [dict(type="attention", mixer=att, mlp=dense), dict(type="attention", mixer=att, mlp=moe),
+              dict(type="latent_attention", mixer=latent, mlp=dense), dict(type="attention", mixer=att, mlp=moe),
+              dict(type="attention", mixer=att, mlp=dense), dict(type="attention", mixer=att, mlp=moe)]
+    return dict(architecture="Dovisun", vocab=DESIGN_VOCAB, width=W, norm=dict(eps=1e-5), layers=layers[:max(4, L - 2)],
+                embedding=dict(scale=float(W) ** 0.5), logit_softcap=30.0, loop=dict(start=2, stop=4, times=2))
+
+
 def design_run(args):
-    """Decode at batch 1 / 8 / 64 (1024-token prompts) and one 2048-token prompt, for both designs of a shape."""
+    """Decode at batch 1 / 8 / 64 (1024-token prompts) and one 2048-token prompt, for the designs of a shape."""
     out = {"metric": f"decode and prefill tok/s, designs beside Qwen3 at shape {args.design}, random weights",
            "unit": "tokens/s", "dtype": args.dtype, "data": "synthetic", "shape": args.design, "designs": {}}
-    for label, config in zip(("pamopel", "qwen3", "ziferax"), design_configs(args.design) + (ziferax_config(args.design),)):
-        if args.design_model not in ("both", "all", label) or (label == "ziferax" and args.design_model == "both"):
+    configs = design_configs(args.design) + (ziferax_config(args.design), dovisun_config(args.design))
+    for label, config in zip(("pamopel", "qwen3", "ziferax", "dovisun"), configs):
+        if args.design_model not in ("both", "all", label) or (label in ("ziferax", "dovisun") and args.design_model == "both"):
             continue
         m = Sized(label, args.dtype, 4096, eager=args.eager, config=config)
         rec = {"weights_GB": round(m.wbytes / 1e9, 3), "decode": {}}
-        for batch in (1, 8, 64):
+        # for profiles: --prefill-only T times the prompt alone, --no-points the decode steps at --batch alone
+        for batch in () if args.prefill_only else (args.batch,) if args.no_points else (1, 8, 64):
             tok_s, ms, _, ctx = m.decode(batch, args.steps, args.warmup, 1024)
             rec["decode"][f"b{batch}"] = {"tok_s": round(tok_s, 1), "ms_per_step": round(ms, 3), "context": round(ctx)}
-        p_tok_s, p_ms, _ = m.prefill(2048)
-        rec["prefill_2048"] = {"tok_s": round(p_tok_s, 1), "ms": round(p_ms, 3)}
+        if not args.no_points or args.prefill_only:
+            n = args.prefill_only or 2048
+            p_tok_s, p_ms, _ = m.prefill(n)
+            rec[f"prefill_{n}"] = {"tok_s": round(p_tok_s, 1), "ms": round(p_ms, 3)}
         out["designs"][label] = rec
         m.close()
     print(json.dumps(out))

@@ -88,10 +88,10 @@ def latent_attention(w, prefix: str, m: dict, eps: float, h: torch.Tensor) -> to
     pos = torch.arange(T)
     cq = rms(h @ w[f"{prefix}.dq"].T, eps) * w[f"{prefix}.dq.norm"]
     q = (cq @ w[f"{prefix}.uq"].T).view(T, H, d + r)
-    q_plain, q_rot = q[..., :d], rotate_halves(q[..., d:], pos, m["rot"])
+    q_plain, q_rot = q[..., :d], rotate_halves(q[..., d:], pos, m["rot"]) if r else q[..., d:]
     down = h @ w[f"{prefix}.dkv"].T
     c = rms(down[:, :kr], eps) * w[f"{prefix}.dkv.norm"]
-    k_rot = rotate_halves(down[:, kr:], pos, m["rot"])                     # one for all heads
+    k_rot = rotate_halves(down[:, kr:], pos, m["rot"]) if r else down[:, kr:]   # one for all heads
     k_plain = (c @ w[f"{prefix}.uk"].T).view(T, H, d)
     v = (c @ w[f"{prefix}.uv"].T).view(T, H, dv)
     gate = torch.sigmoid(h @ w[f"{prefix}.g"].T)                           # [T, H]
@@ -112,10 +112,17 @@ def expert(w, prefix: str, h: torch.Tensor) -> torch.Tensor:
     return (g * torch.sigmoid(g) * (h @ w[f"{prefix}.up"].T)) @ w[f"{prefix}.down"].T
 
 
+MARGINS = None      # a list: every routed layer run appends, per row, the gap between the last chosen logit and the next
+
+
 def route(w, prefix: str, f: dict, h: torch.Tensor):
     """(chosen experts long [T, top], their weights [T, top], logits [T, experts])."""
     z = h @ w[f"{prefix}.router"].T + w[f"{prefix}.router.b"]
     top = torch.topk(z, f["router"]["top"], dim=-1)
+    if MARGINS is not None:
+        ranked = torch.sort(z, dim=-1, descending=True).values
+        k = f["router"]["top"]
+        MARGINS.append((ranked[:, k - 1] - ranked[:, k]) if k < z.shape[-1] else torch.full((z.shape[0],), math.inf))
     return top.indices, torch.softmax(top.values, -1), z
 
 

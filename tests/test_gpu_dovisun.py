@@ -1,0 +1,599 @@
+"""Dovisun in the framework against the plain implementation (``plain_dovisun``, 64-bit): each mechanism's kernels
+alone and as one-layer models; the stream after every layer run; whole prompts; a prompt and then token by token,
+also from the very first token; portions down to two tokens; unequal requests in one batch against each alone, in a
+pool and slots that are used again; scores scaled so that single keys, hundreds of tokens back or beside a page's
+border, decide a row; the softmax's one more term where it outweighs the keys; routers whose top count and bias take
+every special value; long decoding through captured steps; sizes that differ wherever they can; greedy generation
+through the entry point.  In 32-bit to rounding; in bfloat16, where a rounded router input may choose another expert
+at a close call, most rows to rounding and every row within a bound that a lost key or a stale slot exceeds."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+from safetensors.torch import save_file
+
+import plain_dovisun as plain
+from gpu_util import DEV
+
+pytestmark = pytest.mark.gpu
+
+REL = {"float32": 2e-5, "bfloat16": 3e-2}
+
+
+def att(heads, kv, dim, vdim, scale, mlp=None):
+    return dict(type="attention", mixer=dict(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, scale=scale), mlp=mlp)
+
+
+def lat(heads, dim, rot, vdim, q_rank, kv_rank, scale, base=10000.0, scaling=(4.0, 32, 8.0, 1.0), mlp=None):
+    mixer = dict(heads=heads, dim=dim, rot_dim=rot, vdim=vdim, q_rank=q_rank, kv_rank=kv_rank, scale=scale)
+    if rot:
+        mixer["rot"] = dict(base=base, dims=rot)
+        if scaling:
+            mixer["rot"]["scaling"] = dict(factor=scaling[0], original=scaling[1], fast=scaling[2], slow=scaling[3])
+    return dict(type="latent_attention", mixer=mixer, mlp=mlp)
+
+
+def dense(ff):
+    return dict(kind="dense", ff=ff)
+
+
+def moe(experts, top, ff):
+    return dict(kind="moe", router=dict(experts=experts, top=top), expert=dict(ff=ff))
+
+
+def config(width, vocab, layers, loop=None, eps=1e-5, scale=None, cap=None):
+    out = dict(architecture="Dovisun", vocab=vocab, width=width, layers=layers, norm=dict(eps=eps))
+    if loop:
+        out["loop"] = dict(start=loop[0], stop=loop[1], times=loop[2])
+    if scale is not None:
+        out["embedding"] = dict(scale=scale)
+    if cap is not None:
+        out["logit_softcap"] = cap
+    return out
+
+
+# A: the usual shape: the two middle layers (an attention layer with experts, a latent layer) are passed twice
+CFG_A = config(64, 97, [att(4, 2, 32, 32, 0.2, dense(96)), att(6, 2, 16, 24, 0.3, moe(6, 2, 24)),
+                        lat(4, 16, 8, 24, 24, 40, 0.2, mlp=dense(80)), att(2, 1, 64, 64, 0.15, moe(4, 1, 32))],
+               loop=(1, 3, 2), scale=8.0, cap=12.0)
+# B: sizes that differ wherever they can: no loop, no cap and no embedding scale; heads stored padded (24 as 32), as
+# many key heads as query heads, one head; values wider and narrower than keys; a latent layer without rotated dims
+# and one whose rotation is not stretched; every expert chosen (top = all), one expert alone, a layer without a
+# feed-forward, an expert size that no 16-byte access fits
+CFG_B = config(40, 131, [att(3, 3, 24, 10, 0.3, moe(3, 3, 12)), lat(1, 12, 0, 20, 7, 18, 0.25), att(1, 1, 16, 40, 0.25, dense(24)),
+                         lat(5, 6, 10, 4, 30, 9, 0.3, base=500.0, scaling=None, mlp=moe(1, 1, 20)),
+                         att(5, 1, 8, 8, 0.4, moe(7, 1, 6))], eps=1e-3)
+# C: head sizes the matrix-core kernels take (128, 64 and a latent of 104 + 24 kept as one head of 128, one of 200 +
+# 56 as 256), expert sizes the matrix-core products take, many experts, the whole stack passed three times
+CFG_C = config(128, 113, [att(4, 1, 128, 128, 0.09, moe(24, 4, 32)), lat(4, 32, 24, 48, 48, 104, 0.13, base=1e6, scaling=(8.0, 64, 32.0, 1.0), mlp=dense(256)),
+                          att(8, 2, 64, 64, 0.12, dense(136)), lat(2, 64, 56, 64, 64, 200, 0.09, mlp=moe(8, 2, 64))],
+               loop=(0, 4, 3), scale=3.0, cap=20.0)
+# S: scores of many units, so that a softmax row is nearly one key: unit-norm heads give q . k up to the head size,
+# latent heads the same through large scales; the first layer alone is passed twice
+CFG_S = config(32, 1200, [att(2, 1, 16, 16, 2.5, dense(32)), lat(2, 8, 8, 12, 12, 24, 0.6, base=100.0, scaling=(16.0, 64, 4.0, 1.0)),
+                        att(2, 2, 32, 8, 1.5, moe(2, 1, 16))], loop=(0, 1, 2), scale=4.0)
+# K: scores that lie far below zero for many rows, so that the one more term outweighs the keys
+CFG_K = config(32, 50, [att(4, 2, 16, 16, 0.5, moe(3, 2, 8))], loop=(0, 1, 1), cap=8.0)
+# one mechanism a model
+CFG_ATT = config(48, 60, [att(6, 3, 24, 20, 0.25)])
+CFG_LAT = config(48, 60, [lat(3, 20, 12, 28, 16, 36, 0.2)])
+CFG_DENSE = config(48, 60, [att(1, 1, 8, 8, 0.1, dense(100))])
+CFG_MOE = config(48, 60, [att(1, 1, 8, 8, 0.1, moe(9, 3, 20))])
+MODELS = {"A": (CFG_A, 1, {}), "B": (CFG_B, 2, {}), "C": (CFG_C, 3, {}), "S": (CFG_S, 4, {}), "K": (CFG_K, 5, {}),
+          "att": (CFG_ATT, 6, {}), "lat": (CFG_LAT, 7, {}), "dense": (CFG_DENSE, 8, {}), "moe": (CFG_MOE, 9, {})}
+
+
+def made_weights(name):
+    cfg, seed, kw = MODELS[name]
+    w = plain.random_weights(cfg, seed, **kw)
+    if name == "K":
+        # keys that point against the queries: the key matrix is the query matrix's negative for half of the heads
+        w["l0.mix.k"][:16] = -w["l0.mix.q"][:16]
+    return w
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    """{name: (folder, config, 64-bit weights)}; the folders hold bfloat16 tensors under the design's names."""
+    out = {}
+    for name, (cfg, _, _) in MODELS.items():
+        d = tmp_path_factory.mktemp(f"dovisun{name}")
+        w = made_weights(name)
+        with open(os.path.join(d, "config.json"), "w") as f:
+            json.dump(cfg, f)
+        save_file({k: v.contiguous() for k, v in w.items()}, os.path.join(d, "model.safetensors"))
+        out[name] = (str(d), cfg, {k: v.double() for k, v in w.items()})
+    return out
+
+
+_oracle_cache = {}
+
+
+def oracle(models, name, toks):
+    return oracle_and_gaps(models, name, toks)[0]
+
+
+def oracle_and_gaps(models, name, toks):
+    """(logits [T, vocab], for every row the smallest gap between its last chosen router logit and the next, over all
+    routed layer runs)."""
+    key = (name, tuple(toks))
+    if key not in _oracle_cache:
+        _, cfg, w = models[name]
+        plain.MARGINS = []
+        logits = plain.forward(w, cfg, list(toks)).float().numpy()
+        gaps = np.min([m.numpy() for m in plain.MARGINS], axis=0) if plain.MARGINS else np.full(len(toks), np.inf)
+        plain.MARGINS = None
+        _oracle_cache[key] = (logits, gaps)
+    return _oracle_cache[key]
+
+
+# bfloat16 bounds (median, 85th of 100 rows, largest row).  A router that reads a rounded input picks another expert
+# where two logits lie closer than rounding moves them: such a row moves as a whole, and the rows that attend to it a
+# little.  So most rows are held to rounding, and every row whose own logits are CLOSE_CALL or more apart to a bound
+# that a lost key or a stale slot exceeds on peaked rows.  Model C runs twelve layers, six of them routed with four of
+# 24 experts: half of its rows have a close call somewhere.
+BF16_BOUNDS = {"C": (3e-2, 8e-2, 0.3)}
+CLOSE_CALL = 0.05
+
+
+def close(got, want, dtype, name="", gaps=None):
+    err = np.abs(got - want).max(-1) / float(np.abs(want).max())
+    if dtype == "float32":
+        assert err.max() <= REL[dtype], f"max {err.max():.3e} at row {int(err.argmax())}"
+        return
+    mid, most, top = BF16_BOUNDS.get(name, (2e-2, REL[dtype], 0.3))
+    clear = err if gaps is None else err[gaps >= CLOSE_CALL]
+    if len(err) >= 8:
+        assert np.median(err) <= mid and np.quantile(err, 0.85) <= most, \
+            f"median {np.median(err):.3e}, 85th {np.quantile(err, 0.85):.3e}"
+    elif len(clear):
+        assert np.median(clear) <= most, f"median {np.median(clear):.3e}"
+    assert not len(clear) or clear.max() <= top, f"max {clear.max():.3e} at row {int(err.argmax())}"
+
+
+def agree(models, name, toks, got, dtype, rows=None):
+    want, gaps = oracle_and_gaps(models, name, toks)
+    if rows is not None:
+        want, gaps = want[rows], gaps[rows]
+    close(got, want, dtype, name, gaps)
+
+
+def tokens(vocab, n, seed):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+@pytest.fixture(scope="module")
+def replayers(models):
+    from ullm_amd.replay import Replayer
+    made = {}
+
+    def get(name, dtype, max_tokens=512, max_requests=4, use_graphs=True):
+        key = (name, dtype, max_tokens, max_requests, use_graphs)
+        if key not in made:
+            made[key] = Replayer(models[name][0], dtype, max_tokens, 16, DEV, max_requests=max_requests, use_graphs=use_graphs)
+        rep = made[key]
+        assert not rep.live and rep.runner.cache.num_free_pages() == rep.max_tokens // 16
+        return rep
+    return get
+
+
+def run(rep, rid, toks, cuts, end=True):
+    """Feed ``toks`` in portions of the sizes ``cuts`` (the rest one by one); logits of every position."""
+    got, at, step = [], 0, 0
+    sizes = list(cuts) + [1] * len(toks)
+    while at < len(toks):
+        n = min(sizes[step], len(toks) - at)
+        got.append(rep.step({"step": step, "entries": [{"id": rid, "tokens": toks[at:at + n], "want": list(range(n))}],
+                             "end": [rid] if end and at + n == len(toks) else []}))
+        at, step = at + n, step + 1
+    return np.concatenate(got)
+
+
+CASES = [(n, d) for n in ("A", "B", "C") for d in ("float32", "bfloat16")]
+
+
+@pytest.mark.parametrize("name,dtype", CASES + [(n, d) for n in ("att", "lat", "dense", "moe") for d in ("float32", "bfloat16")])
+def test_whole_prompts(replayers, models, name, dtype):
+    rep = replayers(name, dtype)
+    for i, n in enumerate((1, 2, 15, 16, 17, 75)):
+        toks = tokens(models[name][1]["vocab"], n, 10 + i)
+        agree(models, name, toks, run(rep, "r", toks, [n]), dtype)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_the_stream_after_every_layer_run(models, name):
+    """Run by run in 32-bit, the step ahead of a pass included: the stream after a layer is the stream before it plus
+    the branch that the layer leaves pending."""
+    from ullm_amd.engine.loading import load_model
+    from ullm_amd.engine.runner import ModelRunner, StepEntry
+    from ullm_amd.kernels import ops
+    d, cfg, w = models[name]
+    toks = tokens(cfg["vocab"], 50, 3)
+    want = []
+    plain.forward(w, cfg, toks, want)
+    _, model, env = load_model(d, "float32", DEV, context_len=64)
+    runner = ModelRunner(model, env, page_size=16, num_pages=4, max_requests=1, use_graphs=False)
+    rc = runner.cache.admit("r")
+    assert runner.cache.reserve(rc, len(toks))
+    ctx, _ = runner.build_context([StepEntry(rc, toks, [])])
+    stream, pending = ops.embedding(ctx.token_ids, model.embedding, scale=model.plan.embedding_scale), None
+    ctx.embedded = stream.clone()
+    n_layers, seen = len(cfg["layers"]), 0
+    for block, cache_id in model.run_order:
+        stream, pending = model.blocks[block].forward(stream, pending, ctx, runner.caches.get(cache_id))
+        if block >= n_layers:
+            assert pending is None                                  # the step ahead of a pass leaves a whole stream
+            continue
+        after = (stream + pending.mult * pending.branch).double().cpu()
+        assert (after - want[seen]).abs().max() <= 2e-5 * want[seen].abs().max(), seen
+        seen += 1
+    assert seen == len(want) == len(plain.run_order(cfg))
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_a_prompt_and_then_token_by_token(replayers, models, name, dtype):
+    toks = tokens(models[name][1]["vocab"], 75, 15)
+    for graphs in (True, False):
+        agree(models, name, toks, run(replayers(name, dtype, use_graphs=graphs), "r", toks, [40]), dtype)
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_token_by_token_from_the_first_token(replayers, models, name, dtype):
+    toks = tokens(models[name][1]["vocab"], 45, 16)
+    agree(models, name, toks, run(replayers(name, dtype), "r", toks, []), dtype)
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+@pytest.mark.parametrize("cuts", [(2, 2, 3, 2, 14, 2, 17, 31, 2), (1, 1, 2, 30, 3, 3, 33), (16, 16, 16, 2, 25)])
+def test_portions_of_changing_size(replayers, models, name, dtype, cuts):
+    toks = tokens(models[name][1]["vocab"], 75, 15)
+    got = run(replayers(name, dtype), "r", toks, cuts)
+    agree(models, name, toks, got, dtype)
+    if dtype == "float32":
+        # 32-bit sums are ordered by the row alone: the cutting changes no bit
+        assert np.array_equal(got, run(replayers(name, dtype), "r", toks, [75]))
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_unequal_requests_together_in_pages_and_slots_used_again(replayers, models, name, dtype):
+    """Six requests through two slots and a pool of 128 tokens: portions beside single tokens, a request left out
+    of a step, a request that starts in the slot and pages another has just given back."""
+    rep = replayers(name, dtype, max_tokens=128, max_requests=2)
+    vocab = models[name][1]["vocab"]
+    reqs = {f"q{i}": tokens(vocab, n, 30 + i) for i, n in enumerate((50, 33, 1, 64, 20, 47))}
+    plan = [[("q0", 20), ("q1", 2)], [("q0", 1), ("q1", 31)], [("q0", 29)],          # q1 ends; q0 goes on alone
+            [("q2", 1)], [("q3", 17)], [("q3", 1)], [("q3", 2)], [("q3", 44)],        # q2 and q3 use q1's and q0's slots again
+            [("q4", 3), ("q5", 30)], [("q5", 1)], [("q4", 16), ("q5", 1)], [("q4", 1), ("q5", 15)]]
+    at = {r: 0 for r in reqs}
+    got = {r: [] for r in reqs}
+    for s, entries in enumerate(plan):
+        msg = {"step": s, "entries": [], "end": []}
+        for r, n in entries:
+            msg["entries"].append({"id": r, "tokens": reqs[r][at[r]:at[r] + n], "want": list(range(n))})
+            at[r] += n
+            if at[r] == len(reqs[r]):
+                msg["end"].append(r)
+        out, row = rep.step(msg), 0
+        for r, n in entries:
+            got[r].append(out[row:row + n])
+            row += n
+    assert at == {r: len(t) for r, t in reqs.items()}
+    for r, toks in reqs.items():
+        agree(models, name, toks, np.concatenate(got[r]), dtype)
+    rep.runner.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_pages_that_return(replayers, models, dtype):
+    """190 tokens one by one through captured steps whose contexts pass many pages; a second request then takes the
+    pages the first gave back."""
+    rep = replayers("A", dtype, max_tokens=192)
+    toks = tokens(models["A"][1]["vocab"], 190, 40)
+    agree(models, "A", toks, run(rep, "r", toks, [3]), dtype)
+    other = tokens(models["A"][1]["vocab"], 100, 41)
+    agree(models, "A", other, run(rep, "s", other, [60]), dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cuts", [(330,), (250,), (17, 64, 2, 130, 2, 30), (33, 33, 1, 1, 47, 47, 2, 16)])
+def test_scores_scaled_so_that_single_keys_decide(replayers, models, dtype, cuts):
+    """With scores of many units a softmax row is close to one key among up to 330, in the prompt's portions and for
+    single tokens behind it: a key lost or doubled at a page's or a tile's border or hundreds of tokens back takes a
+    whole value out of the sum."""
+    toks = tokens(models["S"][1]["vocab"], 330, 42)
+    want = oracle(models, "S", toks)
+    got = run(replayers("S", dtype), "r", toks, cuts)
+    if dtype == "float32":
+        close(got, want, dtype)
+    else:
+        # one key's weight moves by percents under bfloat16 rounding of peaked scores
+        err = np.abs(got - want).max(-1) / np.abs(want).max()
+        assert np.median(err) < 3e-2 and err.max() < 0.3, (np.median(err), err.max())
+
+
+def test_single_far_keys_decide_in_the_peaked_model():
+    """The plain implementation itself: in the peaked model many rows give most of their weight to one key, for a
+    good part of them a key more than a hundred tokens back; without that key the logits move by far more than the
+    bounds above."""
+    w = {k: v.double() for k, v in made_weights("S").items()}
+    cfg = MODELS["S"][0]
+    toks = tokens(cfg["vocab"], 330, 42)
+    e = w["embed"][torch.tensor(toks)] * cfg["embedding"]["scale"]
+    x = torch.cat((e, e), -1) @ w["loop.in"].T
+    h = plain.rms(x, cfg["norm"]["eps"]) * w["l0.norm1"]
+    m = cfg["layers"][0]["mixer"]
+    q = plain.rms((h @ w["l0.mix.q"].T).view(330, 2, 16), 1e-5)
+    k = plain.rms((h @ w["l0.mix.k"].T).view(330, 1, 16), 1e-5)
+    s = ((q[:, 0] @ k[:, 0].T) * m["scale"]).masked_fill(~plain.causal(330), -math.inf)
+    p = plain.softmax_one_more(s)[200:]
+    far = p.argmax(-1) < torch.arange(200, 330) - 100
+    assert float((p.max(-1).values > 0.5).float().mean()) > 0.2 and int(far.sum()) >= 10
+    base = plain.forward(w, cfg, toks)
+    short = plain.forward(w, cfg, toks[30:])                    # the first thirty keys gone
+    moved = (short - base[30:]).abs().max(-1).values / base.abs().max()
+    assert float((moved > 0.05).float().mean()) > 0.1
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cuts", [(70,), (30,), (2, 2, 21, 21, 2)])
+def test_the_one_more_term_outweighs_the_keys(replayers, models, dtype, cuts, monkeypatch):
+    toks = tokens(models["K"][1]["vocab"], 70, 43)
+    agree(models, "K", toks, run(replayers("K", dtype), "r", toks, cuts), dtype)
+    # and it matters: with an ordinary softmax the oracle's logits move by percents
+    _, cfg, w = models["K"]
+    with_it = plain.forward(w, cfg, toks)
+    monkeypatch.setattr(plain, "softmax_one_more", lambda s: torch.softmax(s, -1))
+    moved = (plain.forward(w, cfg, toks) - with_it).abs().max() / with_it.abs().max()
+    assert float(moved) > 0.05
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_greedy_generation_through_the_entry_point(models, name):
+    from ullm_amd import LLM, EngineConfig, SamplingParams
+    d, cfg, w = models[name]
+    g = torch.Generator().manual_seed(50)
+    prompts = [torch.randint(0, cfg["vocab"], (n,), generator=g).tolist() for n in (5, 19, 1, 33)]
+    for kw in (dict(), dict(max_num_batched_tokens=12, max_prefill_chunk=5, max_bs=3), dict(enforce_eager=True, disable_async_scheduling=True)):
+        args = dict(model=d, dtype="float32", max_bs=8, context_len=128, page_size=16, num_pages=24, device=DEV)
+        args.update(kw)
+        llm = LLM(EngineConfig(**args))
+        outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=10, ignore_eos=True))
+        for p, o in zip(prompts, outs):
+            assert o.token_ids == plain.greedy_generate(w, cfg, p, 10)
+        llm.engine.runner.cache.check()
+        assert llm.engine.runner.cache.num_free_pages() == 24
+        llm.shutdown()
+
+
+def test_the_trace_program_runs_the_design(models, trace_run):
+    d, cfg, _ = models["A"]
+    toks = tokens(cfg["vocab"], 40, 60)
+    want = oracle(models, "A", toks)
+    tr = trace_run(d, "float32", 128)
+    a = tr.step([("a", toks[:21], [0, 20])])
+    b = tr.step([("a", toks[21:], [18])], end=["a"])
+    tr.close()
+    close(np.concatenate((a, b)), want[[0, 20, 39]], "float32")
+
+
+# ------------------------------------------------------------------------------------------- kernels alone
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,heads,K,N", [(1, 3, 20, 36), (7, 2, 16, 9), (9, 4, 36, 128), (40, 8, 128, 192), (130, 2, 200, 64),
+                                         (200, 5, 104, 130), (3, 1, 1536, 7)])
+def test_a_matrix_per_head(dtype, T, heads, K, N):
+    """y[t, h] = w[h]^T x[t, h] from strided rows into a strided output, against the 64-bit product of the same
+    operands; a row's result is the same bits whatever rows stand beside it (the hand-written kernel's range)."""
+    from ullm_amd.kernels import ops
+    g = torch.Generator().manual_seed(T + K)
+    wide = torch.randn(T, heads, K + 5, generator=g).to(dtype).to(DEV)
+    x = wide[:, :, 3:3 + K]
+    w = (torch.randn(heads, K, N, generator=g) * 0.2).to(dtype).to(DEV)
+    out_wide = torch.full((T, heads, N + 3), 7.0, dtype=dtype, device=DEV)
+    y = ops.head_linear(x, w, out=out_wide[:, :, :N])
+    want = torch.einsum("thk,hkn->thn", x.double().cpu(), w.double().cpu())
+    tol = 2e-5 if dtype == torch.float32 else 1e-2
+    assert (y.double().cpu() - want).abs().max() <= tol * want.abs().max()
+    assert (out_wide[:, :, N:] == 7.0).all()
+    fresh = ops.head_linear(x, w)
+    assert (fresh.double().cpu() - want).abs().max() <= tol * want.abs().max()
+    if T < ops.HEAD_LINEAR_LIBRARY_FROM or dtype == torch.float32:
+        one = ops.head_linear(x[T // 2:T // 2 + 1], w)
+        assert torch.equal(one[0], fresh[T // 2])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,d,r,qr,kr,scaling", [(3, 20, 12, 16, 36, (4.0, 32, 8.0, 1.0)), (1, 12, 0, 7, 18, None),
+                                                     (5, 6, 10, 30, 9, None), (4, 32, 24, 48, 104, (8.0, 64, 32.0, 1.0)),
+                                                     (2, 64, 56, 64, 200, (16.0, 64, 4.0, 1.0))])
+def test_the_latent_layer_s_own_kernels(dtype, heads, d, r, qr, kr, scaling):
+    """The two norms, the key part's rotation and the cache row; the query rows [W_uk[h]^T q_plain | turned q_rot | 0]:
+    against the plain pieces in 64-bit, for tokens at drawn positions of two sequences whose pages are shuffled."""
+    from ullm_amd.kernels import ops
+    from ullm_amd.parts.attention import padded_head_size
+    from ullm_amd.parts.position import Rotary
+    g = torch.Generator().manual_seed(heads * 100 + kr)
+    P, eps, hd = 16, 1e-4, padded_head_size(kr + r)
+    starts, lens = [37, 0], [1, 40]
+    T = sum(lens)
+    rot = dict(base=1000.0, dims=r)
+    if scaling:
+        rot["scaling"] = dict(factor=scaling[0], original=scaling[1], fast=scaling[2], slow=scaling[3])
+    ldg = -(-heads // 8) * 8
+    proj = torch.randn(T, qr + kr + r + heads, generator=g) * 2
+    q_gain, kv_gain = 1 + 0.3 * torch.randn(qr, generator=g), 1 + 0.3 * torch.randn(kr, generator=g)
+    positions = torch.tensor([s + i for s, n in zip(starts, lens) for i in range(n)], dtype=torch.int32)
+    entry = torch.tensor([b for b, n in enumerate(lens) for _ in range(n)], dtype=torch.int32)
+    pages = [-(-(s + n) // P) for s, n in zip(starts, lens)]
+    order = torch.randperm(sum(pages) + 2, generator=g)
+    table = torch.full((2, max(pages)), -1, dtype=torch.int32)
+    table[0, :pages[0]], table[1, :pages[1]] = order[:pages[0]], order[pages[0]:pages[0] + pages[1]]
+    k_pool = torch.zeros(sum(pages) + 2, 1, P, hd, dtype=dtype, device=DEV)
+    v_pool = torch.zeros(sum(pages) + 2, 1, hd, P, dtype=dtype, device=DEV)
+    cos_sin = Rotary.make_table(r, 1000.0, 64, scaling).to(DEV) if r else None
+    cq, gate = ops.latent_prepare(proj.to(DEV), 0, qr, qr, kr, qr + kr, r, qr + kr + r, heads, q_gain.to(DEV), kv_gain.to(DEV), eps,
+                                  cos_sin, positions.to(DEV), entry.to(DEV), table.to(DEV), k_pool, v_pool, P, hd, True, dtype)
+    x = proj.double()
+    tol = 1e-5 if dtype == torch.float32 else 1.6e-2
+    want_cq = plain.rms(x[:, :qr], eps) * q_gain.double()
+    want_c = plain.rms(x[:, qr:qr + kr], eps) * kv_gain.double()
+    want_kr = plain.rotate_halves(x[:, qr + kr:qr + kr + r], positions.long(), rot) if r else x[:, :0]
+    assert (cq.double().cpu() - want_cq).abs().max() <= tol * want_cq.abs().max()
+    assert gate.shape == (T, ldg) and (gate[:, :heads].double().cpu() - x[:, qr + kr + r:]).abs().max() <= tol * x.abs().max()
+    for t in range(T):
+        b, pos = int(entry[t]), int(positions[t])
+        page, off = int(table[b, pos // P]), pos % P
+        row = k_pool[page, 0, off].double().cpu()
+        assert (row[:kr] - want_c[t]).abs().max() <= tol * want_c.abs().max(), t
+        if r:
+            assert (row[kr:kr + r] - want_kr[t]).abs().max() <= tol * want_kr.abs().max(), t
+        assert (row[kr + r:] == 0).all()
+        assert (v_pool[page, 0, :kr, off].double().cpu() - want_c[t]).abs().max() <= tol * want_c.abs().max(), t
+    # the query rows
+    q = torch.randn(T, heads * (d + r), generator=g).to(dtype)
+    w_uk = (torch.randn(heads, d, kr, generator=g) * 0.2).to(dtype)
+    qa = ops.head_linear(q.to(DEV).view(T, heads, d + r)[:, :, :d], w_uk.to(DEV))
+    rows = ops.latent_query(qa, q.to(DEV), d, r, hd, cos_sin, positions.to(DEV)).double().cpu().view(T, heads, hd)
+    qd = q.double().view(T, heads, d + r)
+    want_a = torch.einsum("thd,hdk->thk", qd[:, :, :d], w_uk.double())
+    assert (rows[:, :, :kr] - want_a).abs().max() <= (tol if dtype == torch.float32 else 3e-2) * want_a.abs().max()
+    if r:
+        want_r = plain.rotate_halves(qd[:, :, d:], positions.long(), rot)
+        assert (rows[:, :, kr:kr + r] - want_r).abs().max() <= tol * want_r.abs().max()
+    assert (rows[:, :, kr + r:] == 0).all()
+
+
+@pytest.mark.parametrize("R,top", [(20, 3), (5, 5), (64, 1), (200, 8), (2, 1), (1, 1)])
+def test_the_largest_logits_and_the_softmax_over_them(R, top):
+    from ullm_amd.kernels import ops
+    g = torch.Generator().manual_seed(R)
+    T = 37
+    z = torch.randn(T, R, generator=g) * 3
+    z[3] = 0.0                                                   # every logit equal: the lowest indices win
+    z[4, :] = -1e4
+    z[4, R - 1] = 50.0                                           # one output has all the weight
+    z[5] = -300.0 + torch.randn(R, generator=g)                  # logits far below zero still give weights that sum to one
+    b = torch.randn(R, generator=g)
+    ids, wts = ops.moe_route(z.to(DEV), b.to(DEV), top, mode=ops.ROUTE_TOP_LOGITS)
+    zb = z.double() + b.double()
+    for t in range(T):
+        want = sorted(range(R), key=lambda e: (-float(zb[t, e]), e))[:top]
+        assert ids[t].tolist() == want, t
+        assert (wts[t].double().cpu() - torch.softmax(zb[t, want], 0)).abs().max() < 1e-5
+    # the product, the bias and the choice in one kernel: the same for a row alone and among others
+    H = 72
+    x = torch.randn(T, H, generator=g)
+    wr = torch.randn(R, H, generator=g) * 0.3
+    ids, wts = ops.moe_router(x.to(DEV), wr.to(DEV), b.to(DEV), top, mode=ops.ROUTE_TOP_LOGITS)
+    one_ids, one_wts = ops.moe_router(x[9:10].to(DEV), wr.to(DEV), b.to(DEV), top, mode=ops.ROUTE_TOP_LOGITS)
+    assert torch.equal(one_ids[0], ids[9]) and torch.equal(one_wts[0], wts[9])
+    zb = x.double() @ wr.double().T + b.double()
+    for t in range(T):
+        order = sorted(range(R), key=lambda e: (-float(zb[t, e]), e))
+        gaps = [float(zb[t, order[i]] - zb[t, order[i + 1]]) for i in range(min(top, R - 1))]
+        if gaps and min(gaps) < 1e-4:
+            continue                                             # a close call: either order is right
+        assert ids[t].tolist() == order[:top], t
+        assert (wts[t].double().cpu() - torch.softmax(zb[t, order[:top]], 0)).abs().max() < 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_the_squared_relu_the_cap_and_the_scaled_embedding(dtype):
+    from ullm_amd.kernels import ops
+    g = torch.Generator().manual_seed(2)
+    x = (torch.randn(13, 40, generator=g) * 3).to(dtype)
+    got = ops.activation(x.to(DEV), ops.ACT_RELU2).double().cpu()
+    want = torch.relu(x.double()) ** 2
+    assert (got - want).abs().max() <= (1e-6 if dtype == torch.float32 else 1e-2) * want.abs().max()
+    z = torch.randn(5, 77, generator=g) * 40
+    z[0, :3] = torch.tensor([0.0, 1e4, -1e4])
+    capped = ops.softcap_(z.clone().to(DEV), 15.0).double().cpu()
+    assert (capped - 15.0 * torch.tanh(z.double() / 15.0)).abs().max() <= 1e-5
+    table = torch.randn(30, 24, generator=g).to(dtype)
+    ids = torch.tensor([3, 29, 0, 3], dtype=torch.int32)
+    rows = ops.embedding(ids.to(DEV), table.to(DEV), scale=2.5).double().cpu()
+    assert (rows - table.double()[ids.long()] * 2.5).abs().max() <= 1e-6 * 10
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_the_step_ahead_of_a_pass(dtype):
+    """[stream + pending | embedding output] side by side and the product with the mixing matrix, as the block does
+    it, against 64-bit."""
+    from types import SimpleNamespace
+    from ullm_amd.parts import build_part
+    from ullm_amd.parts.base import PartEnv
+    g = torch.Generator().manual_seed(8)
+    T, H = 11, 40
+    block = build_part("block", "mix_in_embedding", hidden_size=H, weight_name="m")
+    w = (torch.randn(H, 2 * H, generator=g) * 0.2).to(dtype)
+    block.bind({"m": w.to(DEV)}, PartEnv(torch.device(DEV), dtype, 64))
+    stream, e = torch.randn(T, H, generator=g), torch.randn(T, H, generator=g)
+    branch = torch.randn(T, H, generator=g).to(dtype)
+    ctx = SimpleNamespace(embedded=e.to(DEV), dtype=dtype)
+    for pending in (None, branch.to(DEV)):
+        got, left = block.forward(stream.clone().to(DEV), pending, ctx, None)
+        assert left is None and got.dtype == torch.float32
+        x = stream.double() + (branch.double() if pending is not None else 0)
+        both = torch.cat((x, e.double()), -1)
+        if dtype == torch.bfloat16:
+            both = both.bfloat16().double()                      # the product reads rows of the compute dtype
+        want = both @ w.double().T
+        assert (got.double().cpu() - want).abs().max() <= (2e-5 if dtype == torch.float32 else 2e-3) * want.abs().max()
+
+
+@pytest.mark.parametrize("hd,nq,nkv", [(64, 8, 2), (128, 4, 1), (32, 6, 3), (256, 2, 1), (48, 3, 1)])
+def test_attention_with_one_more_term_of_one(hd, nq, nkv):
+    """The bfloat16 attention kernels with a sink of 0 for every head against 64-bit weights e^s / (1 + sum e^s), on
+    the same rounded operands: rows whose scores all lie far below zero (the output nearly vanishes), rows with one
+    score far above it, contexts that end at and beside page and tile borders, one of 1 100 keys; a prompt portion
+    that starts in the middle of a page beside single tokens; the same in the general kernel."""
+    from types import SimpleNamespace
+    from gpu_util import paged_cache, table_tensor
+    from ullm_amd.kernels import ops
+    from ullm_amd.parts import GroupView, StepShape
+    from ullm_amd.parts.attention import plan_attention_step
+    g = torch.Generator().manual_seed(hd + nq)
+    starts, lens = [1130, 31, 64, 200, 0], [1, 1, 1, 45, 33]
+    seqs_k = [torch.randn(s + n, nkv, hd, generator=g).bfloat16().float() for s, n in zip(starts, lens)]
+    seqs_v = [torch.randn(s + n, nkv, hd, generator=g).bfloat16().float() for s, n in zip(starts, lens)]
+    k_pool, v_pool, tables = paged_cache(seqs_k, seqs_v, 16, torch.bfloat16, DEV, fill=0.0)
+    T = sum(lens)
+    q = torch.randn(T, nq, hd, generator=g).bfloat16()
+    scale = 1.5 / math.sqrt(hd)
+    # head 0 of every token: a query against all keys' mean direction, so that every score is far below zero
+    q[:, 0] = -torch.ones(hd).bfloat16() * 3
+    for k in seqs_k:
+        k[:, 0] = (k[:, 0].abs() + 0.5).bfloat16().float()
+    k_pool, v_pool, tables = paged_cache(seqs_k, seqs_v, 16, torch.bfloat16, DEV, fill=0.0)
+    positions = torch.tensor([s + i for s, n in zip(starts, lens) for i in range(n)], dtype=torch.int32, device=DEV)
+    entry = torch.tensor([b for b, n in enumerate(lens) for _ in range(n)], dtype=torch.int32, device=DEV)
+    plan = plan_attention_step(StepShape(tuple(lens), tuple(starts)))
+    plan.arrays = {k: torch.tensor(v, dtype=torch.int32, device=DEV) for k, v in plan.arrays.items()}
+    group = GroupView(table_tensor(tables, DEV), 0, 16, 0)
+    ctx = SimpleNamespace(positions=positions, token_entry=entry)
+    sink = torch.zeros(nq, dtype=torch.float32, device=DEV)
+    general = ops.paged_attention_generic(q.view(T, nq * hd).to(DEV), k_pool, v_pool, positions, entry, group.block_table,
+                                          16, nq, nkv, hd, scale, 0, sink=sink).float().cpu().view(T, nq, hd)
+    results = [general]
+    if ops.attention_mfma_supports(torch.bfloat16, hd, 16, nq, nkv):
+        out = ops.paged_attention(q.view(T, nq * hd).to(DEV), k_pool, v_pool, ctx, group, nq, nkv, hd, scale, 0, plan,
+                                  sink=sink, sink_log2=sink.clone())
+        results.append(out.float().cpu().view(T, nq, hd))
+    t, vanishing = 0, 0
+    for b, (s, n) in enumerate(zip(starts, lens)):
+        for i in range(n):
+            pos = s + i
+            for h in range(nq):
+                kv = h // (nq // nkv)
+                sc = (seqs_k[b][:pos + 1, kv].double() @ q[t, h].double()) * scale
+                p = plain.softmax_one_more(sc[None])[0]
+                vanishing += float(p.sum()) < 1e-3
+                want = p @ seqs_v[b][:pos + 1, kv].double()
+                for res in results:
+                    err = (res[t, h].double() - want).abs().max()
+                    assert err <= 2e-2 * max(1.0, float(want.abs().max())), (b, i, h, float(err))
+            t += 1
+    assert vanishing >= T // 2

@@ -1,4 +1,4 @@
-// Paged grouped-query attention, general form: any head size up to 512, any number of heads and
+// Paged grouped-query attention, general form: any head size up to 1024, any number of heads and
 // groups, any page size, any mix of prompt portions and single decoded tokens, optional window.
 // One block per (token, query head); keys are visited in tiles of the block size in a fixed order
 // that depends only on the token's own position, so the result for a token is the same however
@@ -14,7 +14,7 @@
 #include "common.h"
 
 #define ATT_THREADS 128
-#define ATT_MAX_HD 512
+#define ATT_MAX_HD 1024
 
 template <typename T>
 __global__ void __launch_bounds__(ATT_THREADS)

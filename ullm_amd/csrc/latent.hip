@@ -9,7 +9,7 @@
 // latent cache, and a head's output  sum_j p_j c_j  is taken through W_uv[h] afterwards.
 //
 //   latent_prepare   the two norms, the key part's rotation, the cache write, the gate logits in the compute dtype
-//   head_linear      y[t, h, :] = W[h] x[t, h, :] for a matrix per head (q' from q_plain; values from latent outputs)
+//   head_linear      y[t, h, :] = W[h]^T x[t, h, :] for a matrix per head (q' from q_plain; values from latent outputs)
 //   latent_query     [ q'_h | rotate(q_rot[h]) | 0.. ] per head, the query rows the attention kernels take
 //
 // All arithmetic is 32-bit; T selects the storage type only.  Sums run in an order that depends on the row alone.
@@ -91,52 +91,111 @@ extern "C" int ullm_latent_prepare(const float* proj, int ld, int q_off, int q_r
 }
 
 // ------------------------------------------------------------------ a matrix per head
-// y[t, h, n] = sum_k w[h, n, k] * x[t, h, k]:  x [T, heads, K] with strides (x_st, x_sh, 1), w contiguous
-// [heads, N, K], y [T, heads, N] with strides (y_st, y_sh, 1).  grid (token tiles of HL_TOKENS, heads); the tile's
-// rows lie in shared memory as 32-bit values; a wave takes every fourth output, its lanes stride K, then the wave
-// adds up: an order that depends on the row alone.  A fetched row of w serves all the tile's tokens.
+// y[t, h, n] = sum_k x[t, h, k] * w[h, k, n]:  x [T, heads, K] with strides (x_st, x_sh, 1), w contiguous
+// [heads, K, N] (a row of w holds one input's weights for all outputs, so a wave's loads of a row are one
+// contiguous piece), y [T, heads, N] with strides (y_st, y_sh, 1).  grid (token tiles of HL_TOKENS, heads, chunks
+// of 64 * NV outputs); the tile's rows of x lie in shared memory as 32-bit values; a lane owns NV adjacent
+// outputs, wave j of the four takes k = j, j + 4, ... in rising order, and the four partial sums are added in
+// wave order through shared memory: an order that depends on the row alone.  A fetched row of w serves all the
+// tile's tokens.
 #define HL_TOKENS 8
-template <typename T>
+template <typename T, int NV>
+__device__ __forceinline__ void hl_load(const T* p, bool ok, float (&v)[NV]) {
+  if constexpr (NV == 1) {
+    v[0] = ok ? ld_f32(p) : 0.f;
+  } else if constexpr (sizeof(T) == 2) {
+    const uint32_t u = ok ? *reinterpret_cast<const uint32_t*>(p) : 0u;
+    v[0] = __builtin_bit_cast(float, u << 16);
+    v[1] = __builtin_bit_cast(float, u & 0xffff0000u);
+  } else {
+    const float2 f = ok ? *reinterpret_cast<const float2*>(p) : make_float2(0.f, 0.f);
+    v[0] = f.x;
+    v[1] = f.y;
+  }
+}
+
+template <typename T, int NV>
 __global__ void __launch_bounds__(256)
 head_linear_kernel(const T* __restrict__ x, long long x_st, long long x_sh, const T* __restrict__ w,
                    T* __restrict__ y, long long y_st, long long y_sh, int n_tokens, int N, int K) {
-  extern __shared__ float xs[];                                        // [HL_TOKENS][K]
-  const int t0 = blockIdx.x * HL_TOKENS, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  extern __shared__ float hl_shared[];
+  float* xs = hl_shared;                                               // [HL_TOKENS][K]
+  float* part = hl_shared + (size_t)HL_TOKENS * K;                     // [4][HL_TOKENS][64 * NV]
+  constexpr int CH = 64 * NV;
+  const int t0 = blockIdx.x * HL_TOKENS, h = blockIdx.y, n0 = blockIdx.z * CH;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n_rows = n_tokens - t0 < HL_TOKENS ? n_tokens - t0 : HL_TOKENS;
   for (int i = tid; i < HL_TOKENS * K; i += 256) {
     const int r = i / K, k = i - r * K;
     xs[i] = r < n_rows ? ld_f32(x + (size_t)(t0 + r) * x_st + (size_t)h * x_sh + k) : 0.f;
   }
   __syncthreads();
-  const T* wh = w + (size_t)h * N * K;
-  for (int n = wave; n < N; n += 4) {
-    float acc[HL_TOKENS];
+  const int n = n0 + lane * NV;
+  const bool ok = n < N;                                               // NV == 2 only where N is even: both or none
+  const T* wp = w + (size_t)h * K * N + n;
+  float acc[HL_TOKENS][NV];
 #pragma unroll
-    for (int r = 0; r < HL_TOKENS; ++r) acc[r] = 0.f;
-    for (int k = lane; k < K; k += 64) {
-      const float wv = ld_f32(wh + (size_t)n * K + k);
+  for (int r = 0; r < HL_TOKENS; ++r)
 #pragma unroll
-      for (int r = 0; r < HL_TOKENS; ++r) acc[r] = fmaf(xs[r * K + k], wv, acc[r]);
-    }
+    for (int v = 0; v < NV; ++v) acc[r][v] = 0.f;
+  int k = wave;
+  for (; k + 12 < K; k += 16) {                                        // four rows of w under way
+    float w0[NV], w1[NV], w2[NV], w3[NV];
+    hl_load<T, NV>(wp + (size_t)k * N, ok, w0);
+    hl_load<T, NV>(wp + (size_t)(k + 4) * N, ok, w1);
+    hl_load<T, NV>(wp + (size_t)(k + 8) * N, ok, w2);
+    hl_load<T, NV>(wp + (size_t)(k + 12) * N, ok, w3);
 #pragma unroll
     for (int r = 0; r < HL_TOKENS; ++r) {
-      const float s = wave_sum(acc[r]);
-      if (lane == 0 && r < n_rows) st_f32(y + (size_t)(t0 + r) * y_st + (size_t)h * y_sh + n, s);
+      const float x0 = xs[r * K + k], x1 = xs[r * K + k + 4], x2 = xs[r * K + k + 8], x3 = xs[r * K + k + 12];
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        acc[r][v] = fmaf(x0, w0[v], acc[r][v]);
+        acc[r][v] = fmaf(x1, w1[v], acc[r][v]);
+        acc[r][v] = fmaf(x2, w2[v], acc[r][v]);
+        acc[r][v] = fmaf(x3, w3[v], acc[r][v]);
+      }
     }
+  }
+  for (; k < K; k += 4) {
+    float w0[NV];
+    hl_load<T, NV>(wp + (size_t)k * N, ok, w0);
+#pragma unroll
+    for (int r = 0; r < HL_TOKENS; ++r)
+#pragma unroll
+      for (int v = 0; v < NV; ++v) acc[r][v] = fmaf(xs[r * K + k], w0[v], acc[r][v]);
+  }
+#pragma unroll
+  for (int r = 0; r < HL_TOKENS; ++r)
+#pragma unroll
+    for (int v = 0; v < NV; ++v) part[((size_t)wave * HL_TOKENS + r) * CH + lane * NV + v] = acc[r][v];
+  __syncthreads();
+  for (int o = tid; o < HL_TOKENS * CH; o += 256) {
+    const int r = o / CH, c = o - r * CH;
+    if (r >= n_rows || n0 + c >= N) continue;
+    float s = part[o];
+    s += part[(size_t)HL_TOKENS * CH + o];
+    s += part[(size_t)2 * HL_TOKENS * CH + o];
+    s += part[(size_t)3 * HL_TOKENS * CH + o];
+    st_f32(y + (size_t)(t0 + r) * y_st + (size_t)h * y_sh + n0 + c, s);
   }
 }
 
 extern "C" int ullm_head_linear(const void* x, long long x_st, long long x_sh, const void* w, void* y, long long y_st,
                                 long long y_sh, int T_, int heads, int N, int K, int dtype, hipStream_t stream) {
   if (T_ <= 0) return 0;
-  if (heads < 1 || heads > 65535 || N < 1 || K < 1 || (size_t)K * HL_TOKENS * sizeof(float) > 64 * 1024) return ULLM_ERR_SHAPE;
-  dim3 grid((T_ + HL_TOKENS - 1) / HL_TOKENS, heads), block(256);
-  const size_t lds = (size_t)K * HL_TOKENS * sizeof(float);
-#define GO(TT) hipLaunchKernelGGL(head_linear_kernel<TT>, grid, block, lds, stream, (const TT*)x, x_st, x_sh, (const TT*)w, \
-    (TT*)y, y_st, y_sh, T_, N, K)
-  if (dtype == ULLM_F32) GO(float);
-  else if (dtype == ULLM_BF16) GO(bf16_t);
-  else return ULLM_ERR_DTYPE;
+  if (heads < 1 || heads > 65535 || N < 1 || K < 1 || K > 1536) return ULLM_ERR_SHAPE;      // the rows in shared memory
+  if (dtype != ULLM_F32 && dtype != ULLM_BF16) return ULLM_ERR_DTYPE;
+  // two outputs a lane where a pair is one aligned load and the outputs fill at least a wave that way
+  const int nv = (N % 2 == 0 && N >= 128) ? 2 : 1;
+  const int chunk = 64 * nv;
+  if ((N + chunk - 1) / chunk > 65535) return ULLM_ERR_SHAPE;
+  dim3 grid((T_ + HL_TOKENS - 1) / HL_TOKENS, heads, (N + chunk - 1) / chunk), block(256);
+  const size_t lds = ((size_t)K * HL_TOKENS + (size_t)4 * HL_TOKENS * chunk) * sizeof(float);
+#define GO(TT, NV) hipLaunchKernelGGL((head_linear_kernel<TT, NV>), grid, block, lds, stream, (const TT*)x, x_st, x_sh, \
+    (const TT*)w, (TT*)y, y_st, y_sh, T_, N, K)
+  if (dtype == ULLM_F32) { if (nv == 2) GO(float, 2); else GO(float, 1); }
+  else { if (nv == 2) GO(bf16_t, 2); else GO(bf16_t, 1); }
 #undef GO
   ULLM_LAUNCH_CHECK();
 }

@@ -546,7 +546,7 @@ def paged_attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch
     _check_sink(sink, nq)
     T = q.shape[0]
     _need(q.shape == (T, nq * hd) and q.stride(1) == 1, "q must be [T, nq*hd]")
-    _need(hd <= 512 and nq % nkv == 0, "head_dim > 512 or heads not a multiple of kv heads")
+    _need(hd <= 1024 and nq % nkv == 0, "head_dim > 1024 or heads not a multiple of kv heads")
     _check_pools(k_pool, v_pool, nkv, page_size, hd, q.dtype)
     _i32(positions, "positions", T)
     _i32(token_entry, "token_entry", T)
@@ -1124,18 +1124,31 @@ def latent_prepare(proj: torch.Tensor, q_off: int, q_rank: int, kv_off: int, kv_
     return cq, gate
 
 
+HEAD_LINEAR_MAX_K = 1536          # the widest rows the per-head kernel keeps in shared memory
+HEAD_LINEAR_LIBRARY_FROM = 128    # from this many rows on a bfloat16 product per head is the library's batched product
+
+
 def head_linear(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """y[t, h] = w[h] x[t, h] for x [T, heads, K] (unit stride along K, any strides otherwise), w contiguous
-    [heads, N, K] of x's dtype; y [T, heads, N] (``out`` may be a strided view with unit stride along N).  32-bit sums
-    in an order that depends on the row alone."""
+    """y[t, h] = w[h]^T x[t, h] for x [T, heads, K] (unit stride along K, any strides otherwise), w contiguous
+    [heads, K, N] of x's dtype; y [T, heads, N] (``out`` may be a strided view with unit stride along N; without
+    ``out`` the result may be one).  Few rows, and float32 always, take the hand-written kernel (32-bit sums in an
+    order that depends on the row alone); many bfloat16 rows the library's batched product."""
     T, heads, K = x.shape
-    _need(w.dim() == 3 and w.shape[0] == heads and w.shape[2] == K and w.is_contiguous() and w.dtype == x.dtype,
-          "w must be contiguous [heads, N, K] of x's dtype")
+    _need(w.dim() == 3 and w.shape[0] == heads and w.shape[1] == K and w.is_contiguous() and w.dtype == x.dtype
+          and w.data_ptr() % 8 == 0, "w must be contiguous [heads, K, N] of x's dtype")
     _need(x.stride(2) == 1, "x must have unit stride along K")
-    N = w.shape[1]
+    N = w.shape[2]
+    if out is not None:
+        _need(out.shape == (T, heads, N) and out.stride(2) == 1 and out.dtype == x.dtype, "bad head_linear output")
+    if x.dtype == torch.bfloat16 and T >= HEAD_LINEAR_LIBRARY_FROM and x.is_cuda:
+        y = torch.bmm(x.transpose(0, 1), w).transpose(0, 1)          # [heads, T, N] seen as [T, heads, N]
+        if out is None:
+            return y
+        out.copy_(y)
+        return out
+    _need(K <= HEAD_LINEAR_MAX_K, f"head_linear takes rows of up to {HEAD_LINEAR_MAX_K} values")
     if out is None:
         out = torch.empty((T, heads, N), dtype=x.dtype, device=x.device)
-    _need(out.shape == (T, heads, N) and out.stride(2) == 1 and out.dtype == x.dtype, "bad head_linear output")
     ll = ctypes.c_longlong
     _check(build.load("latent").ullm_head_linear(_p(x), ll(x.stride(0)), ll(x.stride(1)), _p(w), _p(out), ll(out.stride(0)),
                                                  ll(out.stride(1)), _c_int(T), _c_int(heads), _c_int(N), _c_int(K),

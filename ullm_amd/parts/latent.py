@@ -45,11 +45,11 @@ class LatentAttention(Mixer):
         self.hidden_size, self.nq, self.dim, self.rot, self.vdim = hidden_size, num_heads, head_dim, rot_dim, value_dim
         self.q_rank, self.kv_rank, self.scale, self.eps = q_rank, kv_rank, float(scale), float(norm_eps)
         self.hd = padded_head_size(kv_rank + rot_dim)        # the size of the one cached head
-        if self.hd > 512:
-            raise ValueError(f"a latent of {kv_rank} and {rot_dim} rotated dims: the cached head is at most 512")
+        if self.hd > 1024:
+            raise ValueError(f"a latent of {kv_rank} and {rot_dim} rotated dims: the cached head is at most 1024")
         self.prefix, self.position, self.head_gate = prefix, position, bool(head_gate)
         self.names = {**DEFAULT_NAMES, **(names or {})}
-        self.w_down = self.w_uq = self.w_ukT = self.w_uv = self.w_o = self.q_gain = self.kv_gain = None
+        self.w_down = self.w_uq = self.w_uk = self.w_uvT = self.w_o = self.q_gain = self.kv_gain = None
 
     def children(self):
         return [self.position] if self.position is not None else []
@@ -77,9 +77,10 @@ class LatentAttention(Mixer):
         nq, d, dv, kr = self.nq, self.dim, self.vdim, self.kv_rank
         self.w_down = tensors[f"{self.prefix}.down"].contiguous()
         self.w_uq = tensors[self._name("uq")].contiguous()
-        # per head the matrix that takes the plain query dims to the latent: W_uk[h]^T, stored [heads, kv_rank, dim]
-        self.w_ukT = tensors[self._name("uk")].view(nq, d, kr).transpose(1, 2).contiguous()
-        self.w_uv = tensors[self._name("uv")].contiguous().view(nq, dv, kr)
+        # a matrix per head, stored [heads, inputs, outputs]: W_uk[h] as it is takes the plain query dims to the
+        # latent (q' = W_uk[h]^T q_plain), W_uv[h] transposed takes a latent to the head's values
+        self.w_uk = tensors[self._name("uk")].contiguous().view(nq, d, kr)
+        self.w_uvT = tensors[self._name("uv")].view(nq, dv, kr).transpose(1, 2).contiguous()
         self.w_o = tensors[self._name("o")].contiguous()
         self.q_gain = tensors[self._name("dq_norm")].contiguous()
         self.kv_gain = tensors[self._name("dkv_norm")].contiguous()
@@ -96,9 +97,10 @@ class LatentAttention(Mixer):
             self.q_gain, self.kv_gain, self.eps, table, ctx.positions, ctx.token_entry, group.block_table,
             cache.k_pool, cache.v_pool, group.page_size, hd, cache.owner, ctx.dtype)
         q = linear(cq, self.w_uq)                                                   # [T, nq * (d + r)]
-        into_latent = ops.head_linear(q.view(T, nq, d + r)[:, :, :d], self.w_ukT)   # [T, nq, kr]
+        into_latent = ops.head_linear(q.view(T, nq, d + r)[:, :, :d], self.w_uk)    # [T, nq, kr]
         queries = ops.latent_query(into_latent, q, d, r, hd, table, ctx.positions)  # [T, nq * hd]
         out = ops.paged_attention(queries, cache.k_pool, cache.v_pool, ctx, group, nq, 1, hd, self.scale, 0,
                                   ctx.plans["attention"], gate=gate)
-        values = ops.head_linear(out.view(T, nq, hd)[:, :, :kr], self.w_uv)         # [T, nq, dv]
+        values = torch.empty((T, nq, self.vdim), dtype=out.dtype, device=out.device)
+        ops.head_linear(out.view(T, nq, hd)[:, :, :kr], self.w_uvT, out=values)     # [T, nq, dv]
         return linear_into_stream(values.view(T, nq * self.vdim), self.w_o, ctx)

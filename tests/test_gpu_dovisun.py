@@ -383,7 +383,7 @@ def test_the_trace_program_runs_the_design(models, trace_run):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T,heads,K,N", [(1, 3, 20, 36), (7, 2, 16, 9), (9, 4, 36, 128), (40, 8, 128, 192), (130, 2, 200, 64),
-                                         (200, 5, 104, 130), (3, 1, 1536, 7)])
+                                         (200, 5, 104, 130), (3, 1, 1024, 7)])
 def test_a_matrix_per_head(dtype, T, heads, K, N):
     """y[t, h] = w[h]^T x[t, h] from strided rows into a strided output, against the 64-bit product of the same
     operands; a row's result is the same bits whatever rows stand beside it (the hand-written kernel's range)."""
@@ -516,6 +516,22 @@ def test_the_squared_relu_the_cap_and_the_scaled_embedding(dtype):
     ids = torch.tensor([3, 29, 0, 3], dtype=torch.int32)
     rows = ops.embedding(ids.to(DEV), table.to(DEV), scale=2.5).double().cpu()
     assert (rows - table.double()[ids.long()] * 2.5).abs().max() <= 1e-6 * 10
+
+
+def test_the_sum_of_a_block_s_two_branches():
+    """One tensor or a stack of partial sums each, 32-bit or bfloat16, added in 32-bit slice by slice."""
+    from ullm_amd.kernels import ops
+    g = torch.Generator().manual_seed(4)
+    T, H = 19, 40
+    for sa, da in ((0, torch.bfloat16), (3, torch.float32), (0, torch.float32), (2, torch.bfloat16)):
+        for sb, db in ((0, torch.bfloat16), (5, torch.float32), (None, None)):
+            a = torch.randn(*((sa, T, H) if sa else (T, H)), generator=g).to(da)
+            b = None if sb is None else torch.randn(*((sb, T, H) if sb else (T, H)), generator=g).to(db)
+            got = ops.branch_sum(a.to(DEV), None if b is None else b.to(DEV))
+            want = a.float().view(-1, T, H)[0].clone()
+            for piece in list(a.float().view(-1, T, H)[1:]) + ([] if b is None else list(b.float().view(-1, T, H))):
+                want += piece
+            assert got.dtype == torch.float32 and torch.equal(got.cpu(), want)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

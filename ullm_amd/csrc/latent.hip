@@ -95,10 +95,13 @@ extern "C" int ullm_latent_prepare(const float* proj, int ld, int q_off, int q_r
 // [heads, K, N] (a row of w holds one input's weights for all outputs, so a wave's loads of a row are one
 // contiguous piece), y [T, heads, N] with strides (y_st, y_sh, 1).  grid (token tiles of HL_TOKENS, heads, chunks
 // of 64 * NV outputs); the tile's rows of x lie in shared memory as 32-bit values; a lane owns NV adjacent
-// outputs, wave j of the four takes k = j, j + 4, ... in rising order, and the four partial sums are added in
-// wave order through shared memory: an order that depends on the row alone.  A fetched row of w serves all the
-// tile's tokens.
+// outputs, wave j of the HL_WAVES takes k = j, j + HL_WAVES, ... in rising order (eight rows of w under way at a
+// time: few rows are bound by the loads' latency, not their bytes), and the waves' partial sums are added in wave
+// order through shared memory: an order that depends on the row alone.  A fetched row of w serves all the tile's
+// tokens.
 #define HL_TOKENS 8
+#define HL_WAVES 8
+#define HL_THREADS (64 * HL_WAVES)
 template <typename T, int NV>
 __device__ __forceinline__ void hl_load(const T* p, bool ok, float (&v)[NV]) {
   if constexpr (NV == 1) {
@@ -115,17 +118,17 @@ __device__ __forceinline__ void hl_load(const T* p, bool ok, float (&v)[NV]) {
 }
 
 template <typename T, int NV>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(HL_THREADS)
 head_linear_kernel(const T* __restrict__ x, long long x_st, long long x_sh, const T* __restrict__ w,
                    T* __restrict__ y, long long y_st, long long y_sh, int n_tokens, int N, int K) {
   extern __shared__ float hl_shared[];
   float* xs = hl_shared;                                               // [HL_TOKENS][K]
-  float* part = hl_shared + (size_t)HL_TOKENS * K;                     // [4][HL_TOKENS][64 * NV]
-  constexpr int CH = 64 * NV;
+  float* part = hl_shared + (size_t)HL_TOKENS * K;                     // [HL_WAVES][HL_TOKENS][64 * NV]
+  constexpr int CH = 64 * NV, W = HL_WAVES, U = 8;
   const int t0 = blockIdx.x * HL_TOKENS, h = blockIdx.y, n0 = blockIdx.z * CH;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n_rows = n_tokens - t0 < HL_TOKENS ? n_tokens - t0 : HL_TOKENS;
-  for (int i = tid; i < HL_TOKENS * K; i += 256) {
+  for (int i = tid; i < HL_TOKENS * K; i += HL_THREADS) {
     const int r = i / K, k = i - r * K;
     xs[i] = r < n_rows ? ld_f32(x + (size_t)(t0 + r) * x_st + (size_t)h * x_sh + k) : 0.f;
   }
@@ -139,25 +142,20 @@ head_linear_kernel(const T* __restrict__ x, long long x_st, long long x_sh, cons
 #pragma unroll
     for (int v = 0; v < NV; ++v) acc[r][v] = 0.f;
   int k = wave;
-  for (; k + 12 < K; k += 16) {                                        // four rows of w under way
-    float w0[NV], w1[NV], w2[NV], w3[NV];
-    hl_load<T, NV>(wp + (size_t)k * N, ok, w0);
-    hl_load<T, NV>(wp + (size_t)(k + 4) * N, ok, w1);
-    hl_load<T, NV>(wp + (size_t)(k + 8) * N, ok, w2);
-    hl_load<T, NV>(wp + (size_t)(k + 12) * N, ok, w3);
+  for (; k + (U - 1) * W < K; k += U * W) {                            // U rows of w under way
+    float wv[U][NV];
 #pragma unroll
-    for (int r = 0; r < HL_TOKENS; ++r) {
-      const float x0 = xs[r * K + k], x1 = xs[r * K + k + 4], x2 = xs[r * K + k + 8], x3 = xs[r * K + k + 12];
+    for (int u = 0; u < U; ++u) hl_load<T, NV>(wp + (size_t)(k + u * W) * N, ok, wv[u]);
 #pragma unroll
-      for (int v = 0; v < NV; ++v) {
-        acc[r][v] = fmaf(x0, w0[v], acc[r][v]);
-        acc[r][v] = fmaf(x1, w1[v], acc[r][v]);
-        acc[r][v] = fmaf(x2, w2[v], acc[r][v]);
-        acc[r][v] = fmaf(x3, w3[v], acc[r][v]);
+    for (int r = 0; r < HL_TOKENS; ++r)
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const float xv = xs[r * K + k + u * W];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) acc[r][v] = fmaf(xv, wv[u][v], acc[r][v]);
       }
-    }
   }
-  for (; k < K; k += 4) {
+  for (; k < K; k += W) {
     float w0[NV];
     hl_load<T, NV>(wp + (size_t)k * N, ok, w0);
 #pragma unroll
@@ -170,13 +168,12 @@ head_linear_kernel(const T* __restrict__ x, long long x_st, long long x_sh, cons
 #pragma unroll
     for (int v = 0; v < NV; ++v) part[((size_t)wave * HL_TOKENS + r) * CH + lane * NV + v] = acc[r][v];
   __syncthreads();
-  for (int o = tid; o < HL_TOKENS * CH; o += 256) {
+  for (int o = tid; o < HL_TOKENS * CH; o += HL_THREADS) {
     const int r = o / CH, c = o - r * CH;
     if (r >= n_rows || n0 + c >= N) continue;
     float s = part[o];
-    s += part[(size_t)HL_TOKENS * CH + o];
-    s += part[(size_t)2 * HL_TOKENS * CH + o];
-    s += part[(size_t)3 * HL_TOKENS * CH + o];
+#pragma unroll
+    for (int j = 1; j < W; ++j) s += part[(size_t)j * HL_TOKENS * CH + o];
     st_f32(y + (size_t)(t0 + r) * y_st + (size_t)h * y_sh + n0 + c, s);
   }
 }
@@ -184,14 +181,14 @@ head_linear_kernel(const T* __restrict__ x, long long x_st, long long x_sh, cons
 extern "C" int ullm_head_linear(const void* x, long long x_st, long long x_sh, const void* w, void* y, long long y_st,
                                 long long y_sh, int T_, int heads, int N, int K, int dtype, hipStream_t stream) {
   if (T_ <= 0) return 0;
-  if (heads < 1 || heads > 65535 || N < 1 || K < 1 || K > 1536) return ULLM_ERR_SHAPE;      // the rows in shared memory
+  if (heads < 1 || heads > 65535 || N < 1 || K < 1 || K > 1024) return ULLM_ERR_SHAPE;      // the rows in shared memory
   if (dtype != ULLM_F32 && dtype != ULLM_BF16) return ULLM_ERR_DTYPE;
   // two outputs a lane where a pair is one aligned load and the outputs fill at least a wave that way
   const int nv = (N % 2 == 0 && N >= 128) ? 2 : 1;
   const int chunk = 64 * nv;
   if ((N + chunk - 1) / chunk > 65535) return ULLM_ERR_SHAPE;
-  dim3 grid((T_ + HL_TOKENS - 1) / HL_TOKENS, heads, (N + chunk - 1) / chunk), block(256);
-  const size_t lds = ((size_t)K * HL_TOKENS + (size_t)4 * HL_TOKENS * chunk) * sizeof(float);
+  dim3 grid((T_ + HL_TOKENS - 1) / HL_TOKENS, heads, (N + chunk - 1) / chunk), block(HL_THREADS);
+  const size_t lds = ((size_t)K * HL_TOKENS + (size_t)HL_WAVES * HL_TOKENS * chunk) * sizeof(float);
 #define GO(TT, NV) hipLaunchKernelGGL((head_linear_kernel<TT, NV>), grid, block, lds, stream, (const TT*)x, x_st, x_sh, \
     (const TT*)w, (TT*)y, y_st, y_sh, T_, N, K)
   if (dtype == ULLM_F32) { if (nv == 2) GO(float, 2); else GO(float, 1); }
@@ -203,18 +200,18 @@ extern "C" int ullm_head_linear(const void* x, long long x_st, long long x_sh, c
 // ------------------------------------------------------------------ the query rows of the attention kernels
 // out[t, h, :] = [ qa[t, h, 0 .. rank) | rotate(q[t, h, plain .. plain + rot)) | zeros up to hd ]:  qa with strides
 // (qa_st, qa_sh, 1); q [T, heads * (plain + rot)] the up-projected queries, whose last rot dims per head are
-// turned by the token's position (half-split pairs, table as above).  One block per token.
+// turned by the token's position (half-split pairs, table as above).  One block of LQ_THREADS per (token, head).
+#define LQ_THREADS 128
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(LQ_THREADS)
 latent_query_kernel(const T* __restrict__ qa, long long qa_st, long long qa_sh, const T* __restrict__ q, int ldq,
                     int plain, int rot, int rank, int heads, int hd, const float* __restrict__ cos_sin, int table_rows,
                     const int* __restrict__ positions, T* __restrict__ out, int ldo) {
-  const int t = blockIdx.x, tid = threadIdx.x;
+  const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int pos = positions[t], half = rot / 2;
   const int p = pos < table_rows ? pos : table_rows - 1;
   const float* cs = cos_sin + (size_t)p * rot;
-  for (int i = tid; i < heads * hd; i += 256) {
-    const int h = i / hd, d = i - h * hd;
+  for (int d = tid; d < hd; d += LQ_THREADS) {
     float v = 0.f;
     if (d < rank) {
       v = ld_f32(qa + (size_t)t * qa_st + (size_t)h * qa_sh + d);
@@ -224,7 +221,7 @@ latent_query_kernel(const T* __restrict__ qa, long long qa_st, long long qa_sh, 
       if (j < half) v = ld_f32(qr + j) * cs[j] - ld_f32(qr + j + half) * cs[half + j];
       else v = ld_f32(qr + j) * cs[j - half] + ld_f32(qr + j - half) * cs[j];
     }
-    st_f32(out + (size_t)t * ldo + i, v);
+    st_f32(out + (size_t)t * ldo + (size_t)h * hd + d, v);
   }
 }
 
@@ -232,11 +229,11 @@ extern "C" int ullm_latent_query(const void* qa, long long qa_st, long long qa_s
                                  int rot, int rank, int heads, int hd, const float* cos_sin, int table_rows,
                                  const int* positions, void* out, int ldo, int T_, int dtype, hipStream_t stream) {
   if (T_ <= 0) return 0;
-  if (heads < 1 || plain < 0 || rot < 0 || (rot & 1) || rank < 1 || hd < rank + rot || ldq < heads * (plain + rot) ||
-      ldo < heads * hd)
+  if (heads < 1 || heads > 65535 || plain < 0 || rot < 0 || (rot & 1) || rank < 1 || hd < rank + rot ||
+      ldq < heads * (plain + rot) || ldo < heads * hd)
     return ULLM_ERR_SHAPE;
   if (rot > 0 && (!cos_sin || table_rows <= 0)) return ULLM_ERR_SHAPE;
-#define GO(TT) hipLaunchKernelGGL(latent_query_kernel<TT>, dim3(T_), dim3(256), 0, stream, (const TT*)qa, qa_st, qa_sh, \
+#define GO(TT) hipLaunchKernelGGL(latent_query_kernel<TT>, dim3(T_, heads), dim3(LQ_THREADS), 0, stream, (const TT*)qa, qa_st, qa_sh, \
     (const TT*)q, ldq, plain, rot, rank, heads, hd, cos_sin, table_rows, positions, (TT*)out, ldo)
   if (dtype == ULLM_F32) GO(float);
   else if (dtype == ULLM_BF16) GO(bf16_t);

@@ -185,6 +185,22 @@ def residual_add(branch: torch.Tensor, residual: torch.Tensor) -> None:
                                  _stream()), "residual_add")
 
 
+def branch_sum(a: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 [T, H]: the sum of two branches, each one tensor [T, H] or a stack of partial sums [S, T, H]
+    (contiguous, float32 or bfloat16), added slice by slice, ``a``'s first; ``b`` None: ``a``'s slices alone."""
+    shape = tuple(a.shape[-2:])
+    for t in (a, b):
+        _need(t is None or (t.is_contiguous() and t.dim() in (2, 3) and tuple(t.shape[-2:]) == shape),
+              "branch_sum takes contiguous [T, H] or [S, T, H] of one row shape")
+    out = torch.empty(shape, dtype=torch.float32, device=a.device)
+    sa = a.shape[0] if a.dim() == 3 else 1
+    sb = 0 if b is None else (b.shape[0] if b.dim() == 3 else 1)
+    _check(build.load("elementwise").ullm_branch_sum(_p(a), _c_int(sa), _c_int(_dt(a)), _p(b), _c_int(sb),
+                                                     _c_int(_dt(b) if b is not None else F32), _p(out),
+                                                     ctypes.c_longlong(out.numel()), _stream()), "branch_sum")
+    return out
+
+
 def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
     """y [T, N] += bias (float32 [N]) in place, the sum taken in 32-bit; returns y."""
     T, N = y.shape
@@ -1124,7 +1140,7 @@ def latent_prepare(proj: torch.Tensor, q_off: int, q_rank: int, kv_off: int, kv_
     return cq, gate
 
 
-HEAD_LINEAR_MAX_K = 1536          # the widest rows the per-head kernel keeps in shared memory
+HEAD_LINEAR_MAX_K = 1024          # the widest rows the per-head kernel keeps in shared memory
 HEAD_LINEAR_LIBRARY_FROM = 128    # from this many rows on a bfloat16 product per head is the library's batched product
 
 

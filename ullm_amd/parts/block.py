@@ -109,7 +109,7 @@ class SandwichBlock(Block):
 
 def _one_branch(y):
     """A stack of partial sums [S, T, hidden] added up: a norm behind the branch needs the whole rows."""
-    return y.sum(0).contiguous() if y.dim() == 3 else y
+    return ops.branch_sum(y) if y.dim() == 3 else y
 
 
 @register_part("block", "parallel")
@@ -136,15 +136,13 @@ class ParallelBlock(Block):
         if isinstance(pending, PendingNorm):
             pending = None                               # the stream is complete; this block norms it itself
         h = self.norm.add_norm(pending, residual, out_dtype=ctx.dtype)
-        mixed = _one_branch(self.mixer.forward(h, ctx, cache))
+        mixed = self.mixer.forward(h, ctx, cache)
         if self.ffn is None:
-            return residual, NormedBranch(mixed, None, self.mult)
+            return residual, NormedBranch(_one_branch(mixed), None, self.mult)
         if hasattr(self.ffn, "forward_onto"):
-            return residual, NormedBranch(self.ffn.forward_onto(h, ctx, mixed), None, self.mult)
-        total = torch.zeros(mixed.shape, dtype=torch.float32, device=mixed.device)
-        ops.residual_add(mixed, total)
-        ops.residual_add(_one_branch(self.ffn.forward(h, ctx)), total)
-        return residual, NormedBranch(total, None, self.mult)
+            return residual, NormedBranch(self.ffn.forward_onto(h, ctx, _one_branch(mixed)), None, self.mult)
+        # one kernel adds the two branches, whichever of them are stacks of partial sums
+        return residual, NormedBranch(ops.branch_sum(mixed, self.ffn.forward(h, ctx)), None, self.mult)
 
 
 @register_part("block", "mix_in_embedding")

@@ -518,6 +518,37 @@ def test_the_squared_relu_the_cap_and_the_scaled_embedding(dtype):
     assert (rows - table.double()[ids.long()] * 2.5).abs().max() <= 1e-6 * 10
 
 
+@pytest.mark.parametrize("M", [1, 9, 40, 64, 100, 300])
+@pytest.mark.parametrize("kind", ["relu2", "gelu_tanh"])
+def test_an_ungated_activation_on_store_of_the_products(M, kind):
+    """act(x W^T + b) on the 32-bit sums inside the few-rows and rows kernels, and behind the library's product for
+    more rows, against 64-bit products of the same operands."""
+    from ullm_amd.kernels import ops
+    g = torch.Generator().manual_seed(M)
+    K, N = 256, 192
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.15).bfloat16()
+    b = torch.randn(N, generator=g).float()
+    act = ops.ACT_RELU2 if kind == "relu2" else ops.ACT_GELU_TANH
+
+    def f(z):
+        return torch.relu(z) ** 2 if kind == "relu2" else 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
+    for bias in (None, b):
+        z = x.double() @ w.double().T + (bias.double() if bias is not None else 0)
+        got = [ops.gemm_bf16(x.to(DEV), w.to(DEV), None if bias is None else bias.to(DEV), act=act)]
+        if M <= 64:
+            got.append(ops.gemm_skinny(x.to(DEV), w.to(DEV), None if bias is None else bias.to(DEV), act=act))
+            got.append(ops.gemm_skinny(x.to(DEV), w.to(DEV), None if bias is None else bias.to(DEV), out_dtype=torch.float32, act=act))
+        if ops.gemm_rows_supports(x.to(DEV), w.to(DEV)):
+            got.append(ops.gemm_rows(x.to(DEV), w.to(DEV), None if bias is None else bias.to(DEV), act=act))
+        for out in got:
+            tol = 1e-2 if out.dtype == torch.bfloat16 else 1e-4
+            assert (out.double().cpu() - f(z)).abs().max() <= tol * f(z).abs().max()
+    # and the same product without it is unchanged
+    plain_out = ops.gemm_bf16(x.to(DEV), w.to(DEV))
+    assert (plain_out.double().cpu() - x.double() @ w.double().T).abs().max() <= 1e-2 * (x.double() @ w.double().T).abs().max()
+
+
 def test_the_sum_of_a_block_s_two_branches():
     """One tensor or a stack of partial sums each, 32-bit or bfloat16, added in 32-bit slice by slice."""
     from ullm_amd.kernels import ops

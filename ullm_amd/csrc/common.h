@@ -45,6 +45,19 @@ __device__ __forceinline__ float gated_unit(float g, float u, float limit, float
   return fast_silu(g) * u;
 }
 
+// Activations of an ungated feed-forward on a 32-bit value.  ACT_RELU2: max(x, 0)^2.  ACT_GELU_TANH:
+// 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))).  The product kernels' plain epilogues take ``act`` = kind + 1
+// (0: none) and apply it on store.
+enum { ACT_RELU2 = 0, ACT_GELU_TANH = 1 };
+__device__ __forceinline__ float activate(float x, int kind) {
+  if (kind == ACT_RELU2) {
+    const float r = fmaxf(x, 0.f);
+    return r * r;
+  }
+  return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+}
+__device__ __forceinline__ float activate_on_store(float x, int act) { return act ? activate(x, act - 1) : x; }
+
 __device__ __forceinline__ float ld_f32(const float* p) { return *p; }
 __device__ __forceinline__ float ld_f32(const bf16_t* p) { return bf16_bits_to_f32(*p); }
 __device__ __forceinline__ void st_f32(float* p, float v) { *p = v; }

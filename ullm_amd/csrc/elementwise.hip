@@ -410,16 +410,7 @@ extern "C" int ullm_add_bias(void* y, const float* bias, int T_, int N, long lon
 
 // ------------------------------------------------------------------ activations of an ungated feed-forward
 // out = act(x) element by element on 32-bit values.  ACT_RELU2: max(x, 0)^2.  ACT_GELU_TANH:
-// 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))).
-enum { ACT_RELU2 = 0, ACT_GELU_TANH = 1 };
-__device__ __forceinline__ float activate(float x, int kind) {
-  if (kind == ACT_RELU2) {
-    const float r = fmaxf(x, 0.f);
-    return r * r;
-  }
-  return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
-}
-
+// 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) (``activate`` of common.h).
 template <typename T>
 __global__ void activation_kernel(const T* __restrict__ x, T* __restrict__ out, size_t total, int kind) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

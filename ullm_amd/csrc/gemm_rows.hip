@@ -42,6 +42,7 @@ struct RowSquares {
   int quads;
   float eps;
   float unit_limit, unit_alpha;       // ROWS_SILU: the gated unit's parameters (limit 0: silu(gate) * up), see gated_unit
+  int act;                            // ROWS_STORE: an ungated activation on store (kind + 1, 0: none), see activate_on_store
 };
 
 #define ROWS_SQ_HELD 8   // groups of four partial sums of squares a lane fetches before the product starts
@@ -226,7 +227,7 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if (EPI == ROWS_SILU) v[j] = gated_unit(acc[0][t][j], acc[NTW - 1][t][j], before.unit_limit, before.unit_alpha);
-      else v[j] = acc[0][t][j] + (bias && nn + j < n_end ? bias[nn + j] : 0.f);
+      else v[j] = activate_on_store(acc[0][t][j] + (bias && nn + j < n_end ? bias[nn + j] : 0.f), before.act);
     }
     bf16_t* cp = C + (size_t)m * ldc + nn;
     if (nn + 3 < n_end) {
@@ -336,14 +337,15 @@ extern "C" int ullm_gemm_rows_supports(int M, int N, int K, int ldx, int ldw, in
 // rsqrt(sum of row_sq[m][.] / K + eps) before the epilogue.
 extern "C" int ullm_gemm_rows(const void* X, int ldx, const void* W, int ldw, const float* bias, void* C, int ldc,
                               int M, int N, int K, int epi, const float* row_sq, int sq_parts, float eps,
-                              float unit_limit, float unit_alpha, hipStream_t stream) {
+                              float unit_limit, float unit_alpha, int act, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (!ullm_gemm_rows_supports(M, N, K, ldx, ldw, ldc, epi)) return ULLM_ERR_SHAPE;
   if (((uintptr_t)X & 15) || ((uintptr_t)W & 15) || ((uintptr_t)C & 7)) return ULLM_ERR_SHAPE;
   if (epi == ROWS_SILU && bias) return ULLM_ERR_UNSUPPORTED;
   if (row_sq && (M > 16 || sq_parts < 4 || sq_parts % 4 || ((uintptr_t)row_sq & 15))) return ULLM_ERR_UNSUPPORTED;
   if (unit_limit > 0.f && epi != ROWS_SILU) return ULLM_ERR_UNSUPPORTED;
-  const RowSquares before{row_sq, sq_parts / 4, eps, unit_limit, unit_alpha};
+  if (act < 0 || act > 2 || (act && epi != ROWS_STORE)) return ULLM_ERR_UNSUPPORTED;
+  const RowSquares before{row_sq, sq_parts / 4, eps, unit_limit, unit_alpha, act};
   const int mt = rows_tiles(M);
   RowsShape s;
   rows_shape(N, mt, epi, rows_compute_units(), &s);

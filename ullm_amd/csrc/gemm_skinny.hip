@@ -64,6 +64,7 @@ struct RowSquares {
   const float* sq;
   int quads;
   float unit_limit, unit_alpha;       // EPI_SILU: the gated unit's parameters (limit 0: silu(gate) * up), see gated_unit
+  int act;                            // EPI_STORE: an ungated activation on store (kind + 1, 0: none), see activate_on_store
 };
 
 
@@ -80,7 +81,8 @@ template <int MT, int NT, int EPI, typename TC, typename RedT>
 __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red, const float* __restrict__ bias,
                                               TC* __restrict__ C, float* __restrict__ R, int ldc, int M, int N, int n0,
                                               bool scaled, const float (*sq)[16 * MT], int K, float eps,
-                                              const NormAhead& ahead, float unit_limit = 0.f, float unit_alpha = 0.f) {
+                                              const NormAhead& ahead, float unit_limit = 0.f, float unit_alpha = 0.f,
+                                              int act = 0) {
   constexpr int OT = EPI == EPI_SILU ? NT / 2 : NT;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   const int g = lane >> 4, r = lane & 15;
@@ -184,7 +186,8 @@ __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red,
       } else {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          if (nn + j < N) st_f32(C + (size_t)m * ldc + nn + j, acc[i][t][j] + (bias ? bias[nn + j] : 0.f));
+          if (nn + j < N)
+            st_f32(C + (size_t)m * ldc + nn + j, activate_on_store(acc[i][t][j] + (bias ? bias[nn + j] : 0.f), act));
       }
     }
   }
@@ -409,7 +412,7 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
   __syncthreads();                                        // the partial sums take the place of the stages
   auto& red = *reinterpret_cast<float (*)[MAXW - 1][NT * MT][64 * 4]>(lds);
   skinny_finish<MT, NT, EPI, TC>(acc, red, bias, C, R, ldc, M, n_end, n0, scaled, sq, K, eps, ahead, before.unit_limit,
-                                 before.unit_alpha);
+                                 before.unit_alpha, before.act);
 }
 
 template <int MT, int NT, int EPI, typename TC, bool NORMX, typename... Args>
@@ -536,7 +539,7 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
                                 int force_waves, const float* gain, float eps, int force_rows,
                                 const float* next_gain, void* next_x, int ld_next, float* next_sq,
                                 const float* row_sq, int sq_parts, float unit_limit, float unit_alpha,
-                                hipStream_t stream) {
+                                int act, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (!ullm_gemm_skinny_supports(M, N, K, ldx, ldw) || ldc < N) return ULLM_ERR_SHAPE;
   if (((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return ULLM_ERR_SHAPE;
@@ -555,7 +558,8 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
             k_per_wave = plan.k_per_wave;
   const NormAhead ahead{next_gain, (bf16_t*)next_x, next_sq, ld_next, (tiles + 3) / 4 * 4};
   if (unit_limit > 0.f && epi != EPI_SILU) return ULLM_ERR_UNSUPPORTED;
-  const RowSquares before{row_sq, sq_parts / 4, unit_limit, unit_alpha};
+  if (act < 0 || act > 2 || (act && epi != EPI_STORE)) return ULLM_ERR_UNSUPPORTED;
+  const RowSquares before{row_sq, sq_parts / 4, unit_limit, unit_alpha, act};
   dim3 grid(tiles), block(64 * waves);
   float* R = (float*)C;
 #define GO_(MT, NT, EPI, TC, NORMX) skinny_launch<MT, NT, EPI, TC, NORMX>(grid, block, stream, X, ldx, \

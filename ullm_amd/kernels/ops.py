@@ -613,7 +613,7 @@ def gemm_skinny_supports(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0, gain=None, eps=0.0, rows=0,
-                 ahead=None, squares=None, unit_limit=0.0, unit_alpha=0.0) -> None:
+                 ahead=None, squares=None, unit_limit=0.0, unit_alpha=0.0, act=0) -> None:
     """``ahead``: (next gain, next x, next squares) that an adding product leaves for the norm after it;
     ``squares``: the [parts, M] sums such a product left, which scale this product's rows."""
     lib = build.load("gemm_skinny")
@@ -624,7 +624,7 @@ def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0, gain=None,
                                 ctypes.c_float(eps), _c_int(rows), _p(next_gain), _p(next_x),
                                 _c_int(next_x.stride(0) if next_x is not None else 0), _p(next_sq), _p(squares),
                                 _c_int(squares.shape[1] if squares is not None else 0), _c_float(unit_limit),
-                                _c_float(unit_alpha), _stream()),
+                                _c_float(unit_alpha), _c_int(act), _stream()),
            "gemm_skinny")
 
 
@@ -638,9 +638,10 @@ def _check_squares(squares: Optional[torch.Tensor], M: int) -> None:
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
                 nt: int = 0, waves: int = 0, rows: int = 0, squares: Optional[torch.Tensor] = None,
-                eps: float = 0.0) -> torch.Tensor:
+                eps: float = 0.0, act: Optional[int] = None) -> torch.Tensor:
     """a [M <= 64, K] times w [N, K] transposed, bfloat16 operands streamed once through the matrix
-    cores, 32-bit accumulation; output bfloat16 or float32.  With ``squares`` (float32 [M <= 16, parts], see
+    cores, 32-bit accumulation; output bfloat16 or float32; ``act`` (ACT_RELU2, ACT_GELU_TANH): that activation of
+    the 32-bit sums (+ bias) on store.  With ``squares`` (float32 [M <= 16, parts], see
     :func:`gemm_skinny_add`) row m of the product is scaled by rsqrt(sum of squares[m] / K + eps) before
     the bias: a is then a stream times a norm's gain and the result the product of the normed stream."""
     M, K = a.shape
@@ -653,7 +654,8 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous(), "bias must be float32 [N]")
     _check_squares(squares, M)
-    _gemm_skinny(a, w, bias, out, M, N, K, 0, _dt(out), nt, waves, eps=float(eps), rows=rows, squares=squares)
+    _gemm_skinny(a, w, bias, out, M, N, K, 0, _dt(out), nt, waves, eps=float(eps), rows=rows, squares=squares,
+                 act=0 if act is None else act + 1)
     return out
 
 
@@ -779,13 +781,15 @@ def gemm_rows_supports(a: torch.Tensor, w: torch.Tensor, silu: bool = False) -> 
 
 def gemm_rows(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, silu: bool = False,
               squares: Optional[torch.Tensor] = None, eps: float = 0.0, limit: float = 0.0,
-              alpha: float = 0.0) -> torch.Tensor:
+              alpha: float = 0.0, act: Optional[int] = None) -> torch.Tensor:
     """a (bfloat16 [M <= 128, K]) times w (bfloat16 [N, K]) transposed (+ bias float32 [N]) as bfloat16 [M, N];
     with ``silu``, w is gate | up [2 I, K] and the result silu(gate) * up [M, I] on the 32-bit sums.  The
     matrix is cut into one block per compute unit and every wave keeps several stages of its rows of w in
     flight: for the row counts between the few-rows kernel and the library.  ``squares``, ``eps``: as in
-    :func:`gemm_skinny`.  With ``silu`` and ``limit`` > 0 the clamped gated unit of :func:`glu_clamped` instead."""
+    :func:`gemm_skinny`.  With ``silu`` and ``limit`` > 0 the clamped gated unit of :func:`glu_clamped` instead;
+    without ``silu``, ``act`` (ACT_RELU2, ACT_GELU_TANH) is applied to the 32-bit sums (+ bias) on store."""
     _need(silu or limit <= 0, "the clamped unit needs gate | up weights")
+    _need(act is None or not silu, "an ungated activation and the gated unit exclude each other")
     M, K = a.shape
     _need(gemm_rows_supports(a, w, silu), "gemm_rows takes bfloat16, M <= 128, K a multiple of 64, N a multiple of 4")
     n_out = w.shape[0] // 2 if silu else w.shape[0]
@@ -799,7 +803,7 @@ def gemm_rows(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
                                                   _c_int(1 if silu else 0), _p(squares),
                                                   _c_int(squares.shape[1] if squares is not None else 0),
                                                   ctypes.c_float(float(eps)), _c_float(float(limit)), _c_float(float(alpha)),
-                                                  _stream()), "gemm_rows")
+                                                  _c_int(0 if act is None else act + 1), _stream()), "gemm_rows")
     return out
 
 
@@ -808,13 +812,23 @@ _MM_TAKES_OUT_DTYPE = "out_dtype" in (torch.mm.__doc__ or "")
 
 
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
-              out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+              out_dtype: Optional[torch.dtype] = None, act: Optional[int] = None) -> torch.Tensor:
     """bfloat16 operands, 32-bit accumulation.  Few rows go to the weight-streaming kernels (up to how many
     for this matrix: :func:`dispatch.limits`), some more, where that was measured to be ahead, to the partial-sums
     kernel and a kernel that adds its stacks; many rows go through the library product (as the reference's
-    linears do, ullm/layers/linear.py:165), which for 32-bit output (logits) stores the accumulator unrounded."""
+    linears do, ullm/layers/linear.py:165), which for 32-bit output (logits) stores the accumulator unrounded.
+    ``act`` (ACT_RELU2, ACT_GELU_TANH): that activation of the result, on store in the few-rows and rows kernels, by
+    the activation kernel behind the others."""
     out_dtype = out_dtype or a.dtype
     M = a.shape[0]
+    if act is not None:
+        lim = dispatch.limits(w.shape[0], w.shape[1])
+        if M <= (lim.f32_skinny if out_dtype == torch.float32 else lim.skinny) and gemm_skinny_supports(a, w):
+            return gemm_skinny(a, w, bias, out_dtype=out_dtype, act=act)
+        if out_dtype == torch.bfloat16 and M <= min(lim.rows, ROWS_MAX_ROWS) and gemm_rows_supports(a, w):
+            return gemm_rows(a, w, bias, act=act)
+        y = gemm_bf16(a, w, bias, out_dtype)
+        return activation(y, act, out=y)
     library = a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.is_cuda
     lim = dispatch.limits(w.shape[0], w.shape[1])
     few = lim.f32_skinny if out_dtype == torch.float32 else lim.skinny

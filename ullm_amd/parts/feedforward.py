@@ -55,7 +55,9 @@ ACTIVATIONS = {"relu2": ops.ACT_RELU2, "gelu_tanh": ops.ACT_GELU_TANH}
 @register_part("ffn", "mlp")
 class MLP(FeedForward):
     """Dense feed-forward without a gate: down(act(up(x))), no biases; ``activation`` is "relu2" (the square of
-    relu) or "gelu_tanh".  The activation is applied to the product as stored (bfloat16 or float32) in 32-bit."""
+    relu) or "gelu_tanh".  The activation is applied in 32-bit: to the product's 32-bit sums on store where the
+    few-rows and rows kernels run, to the stored product (bfloat16 or float32) behind the library's and the 32-bit
+    product."""
 
     def __init__(self, hidden_size: int, intermediate_size: int, prefix: str, activation: str = "relu2",
                  names: Optional[Dict[str, str]] = None):
@@ -75,5 +77,4 @@ class MLP(FeedForward):
         self.w_down = tensors[f"{self.prefix}.{self.names['down']}"].contiguous()
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        up = linear(x, self.w_up)
-        return linear_into_stream(ops.activation(up, self.act, out=up), self.w_down, ctx)
+        return linear_into_stream(linear(x, self.w_up, act=self.act), self.w_down, ctx)

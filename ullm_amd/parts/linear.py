@@ -13,11 +13,14 @@ from ..kernels import dispatch, ops
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-           out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+           out_dtype: Optional[torch.dtype] = None, act: Optional[int] = None) -> torch.Tensor:
+    """``act`` (ops.ACT_RELU2, ops.ACT_GELU_TANH): that activation of the result, on store where the product's
+    kernel has it, by the activation kernel otherwise."""
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32 or weight.dtype == torch.float32:
-        return ops.gemm_simple(x, weight, bias, out_dtype=out_dtype)
-    return ops.gemm_bf16(x, weight, bias, out_dtype=out_dtype)
+        y = ops.gemm_simple(x, weight, bias, out_dtype=out_dtype)
+        return y if act is None else ops.activation(y, act, out=y)
+    return ops.gemm_bf16(x, weight, bias, out_dtype=out_dtype, act=act)
 
 
 def linear_of_norm(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, silu: bool = False) -> torch.Tensor:

@@ -137,9 +137,11 @@ def experts(w, prefix: str, f: dict, h: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def layer(w, cfg: dict, i: int, x: torch.Tensor) -> torch.Tensor:
+def layer(w, cfg: dict, i: int, x: torch.Tensor, round_to=None) -> torch.Tensor:
     L, eps, p = cfg["layers"][i], cfg["norm"]["eps"], f"l{i}"
     h = rms(x, eps) * w[f"{p}.norm1"]
+    if round_to is not None:
+        h = h.to(round_to).to(x.dtype)          # what an engine loses at the least that computes in this type
     if L["type"] == "attention":
         y = attention(w, f"{p}.mix", L["mixer"], eps, h)
     elif L["type"] == "latent_attention":
@@ -164,15 +166,16 @@ def run_order(cfg: dict) -> List[tuple]:
     return order + [(i, False) for i in range(b, n)]
 
 
-def forward(w, cfg: dict, tokens, streams: Optional[list] = None) -> torch.Tensor:
-    """Logits [T, vocab] of one whole sequence; ``streams`` (a list) receives the stream after every layer run."""
+def forward(w, cfg: dict, tokens, streams: Optional[list] = None, round_to=None) -> torch.Tensor:
+    """Logits [T, vocab] of one whole sequence; ``streams`` (a list) receives the stream after every layer run.  With
+    ``round_to`` the sublayers' common input is rounded to that type and nothing else is."""
     ids = torch.as_tensor(tokens, dtype=torch.long)
     e = w["embed"][ids] * (cfg.get("embedding") or {}).get("scale", 1.0)
     x = e
     for i, mix_in in run_order(cfg):
         if mix_in:
             x = torch.cat((x, e), -1) @ w["loop.in"].T
-        x = layer(w, cfg, i, x)
+        x = layer(w, cfg, i, x, round_to)
         if streams is not None:
             streams.append(x)
     z = (rms(x, cfg["norm"]["eps"]) * w["final.norm"]) @ w["head"].T

@@ -195,3 +195,10 @@ def test_what_a_configuration_may_leave_out():
     cfg = DovisunConfig.from_dict(lean)
     assert cfg.embedding_scale == 1.0 and cfg.logit_softcap == 0.0 and not cfg.loops and not cfg.has_loop
     assert cfg.layers[1].mixer.rot_scaling is None
+
+
+def test_the_named_size_for_random_weights():
+    from ullm_amd.config import parse_random_weights
+    d, seed = parse_random_weights("dovisun-2048:5")
+    cfg, model = build_model(d)
+    assert seed == 5 and isinstance(cfg, DovisunConfig) and cfg.loops and len(model.run_order) == 6 + 2 + 2

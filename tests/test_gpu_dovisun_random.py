@@ -9,6 +9,7 @@ import random
 
 import numpy as np
 import pytest
+import torch
 from safetensors.torch import save_file
 
 import plain_dovisun as plain
@@ -137,13 +138,17 @@ def test_drawn_configurations(seed, tmp_path):
     assert np.array_equal(whole, cut), "whole and cut differ in 32-bit"      # 32-bit sums are ordered by the row alone
     for k in reqs:
         assert worst_error(mixed[k][:sharp[k]], want[k][:sharp[k]]) <= bound[k], k
-    # bfloat16: the same schedules.  What rounding does depends on the drawn model (up to twenty layer runs, logits of
-    # a few units; a rounded router input may pick another expert at a close call, and then a row moves), and a prompt
-    # portion and a single token take different product kernels, whose rounding is independent: every schedule is held
-    # to the 64-bit logits, the middle row and 85 rows of 100.  The sharp test of the cutting is the 32-bit one above.
+    # bfloat16: the same schedules.  What rounding does depends on the drawn model (up to twenty layer runs, up to
+    # twelve of them routed: a rounded router input picks another expert at a close call, and then a row moves as a
+    # whole), so the bounds are multiples of what the plain implementation loses when nothing but its sublayers'
+    # inputs are rounded to bfloat16: for the middle row and for 85 rows of 100.  A prompt portion and a single token
+    # take different product kernels, whose rounding is independent, so every schedule is held to the 64-bit logits.
+    # The sharp test of the cutting is the 32-bit one above.
     rng.setstate(state)
     rep = Replayer(str(tmp_path), "bfloat16", 512, 16, DEV, max_requests=4)
     whole, cut, mixed = schedules(rep, rng, reqs)
     for got, k in [(whole, "r0"), (cut, "r0")] + [(mixed[k], k) for k in reqs]:
+        floor = np.abs(plain.forward(wide, cfg, reqs[k], round_to=torch.bfloat16).float().numpy() - want[k]).max(-1) / np.abs(want[k]).max()
+        mid, most = 1e-2 + 4 * float(np.median(floor)), 2e-2 + 4 * float(np.quantile(floor, 0.85))
         err = np.abs(got - want[k]).max(-1) / np.abs(want[k]).max()
-        assert np.median(err) <= 4e-2 and np.quantile(err, 0.85) <= 8e-2, (k, float(np.median(err)), float(np.quantile(err, 0.85)))
+        assert np.median(err) <= mid and np.quantile(err, 0.85) <= most, (k, float(np.median(err)), float(np.quantile(err, 0.85)), mid, most)

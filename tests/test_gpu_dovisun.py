@@ -286,6 +286,29 @@ def test_unequal_requests_together_in_pages_and_slots_used_again(replayers, mode
     rep.runner.cache.check()
 
 
+@pytest.mark.parametrize("name", ["lat", "C"])
+def test_many_single_tokens_in_one_captured_step(replayers, models, name):
+    """140 requests a step, one token each, five steps: the per-head products of the latent layers take the library's
+    batched product from 128 rows on, here inside captured steps that are replayed; against the same steps run
+    eagerly and against the plain implementation."""
+    vocab = models[name][1]["vocab"]
+    reqs = {f"m{i}": tokens(vocab, 5, 200 + i) for i in range(140)}
+    got = {}
+    for graphs in (True, False):
+        rep = replayers(name, "bfloat16", max_tokens=140 * 16, max_requests=140, use_graphs=graphs)
+        rows = {r: [] for r in reqs}
+        for step in range(5):
+            out = rep.step({"step": step, "entries": [{"id": r, "tokens": [t[step]], "want": [0]} for r, t in reqs.items()],
+                            "end": list(reqs) if step == 4 else []})
+            for i, r in enumerate(reqs):
+                rows[r].append(out[i])
+        got[graphs] = {r: np.stack(v) for r, v in rows.items()}
+    for r, toks in reqs.items():
+        assert np.abs(got[True][r] - got[False][r]).max() <= 1e-2 * np.abs(got[False][r]).max(), r
+    for r in list(reqs)[::7]:
+        agree(models, name, reqs[r], got[True][r], "bfloat16")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_and_pages_that_return(replayers, models, dtype):
     """190 tokens one by one through captured steps whose contexts pass many pages; a second request then takes the

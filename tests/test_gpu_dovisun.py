@@ -466,6 +466,7 @@ def test_the_latent_layer_s_own_kernels(dtype, heads, d, r, qr, kr, scaling):
     want_kr = plain.rotate_halves(x[:, qr + kr:qr + kr + r], positions.long(), rot) if r else x[:, :0]
     assert (cq.double().cpu() - want_cq).abs().max() <= tol * want_cq.abs().max()
     assert gate.shape == (T, ldg) and (gate[:, :heads].double().cpu() - x[:, qr + kr + r:]).abs().max() <= tol * x.abs().max()
+    assert (gate[:, heads:] == 0).all()
     for t in range(T):
         b, pos = int(entry[t]), int(positions[t])
         page, off = int(table[b, pos // P]), pos % P

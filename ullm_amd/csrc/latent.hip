@@ -21,7 +21,7 @@
 // gate logits at g_off (n_gate values; n_gate 0: none).
 // Outputs: cq [T, q_rank] = rmsnorm(q latent) * q_gain; key pool row [page, 0, slot, 0 .. kv_rank + rot) and value
 // pool column [page, 0, 0 .. kv_rank, slot] (pools made for one head of size hd >= kv_rank + rot; the dims behind
-// are never written and stay zero); gate [T, ldg] = the gate logits.  Tokens whose page id is negative write no cache.
+// are never written and stay zero); gate [T, ldg] = the gate logits and zeros behind them.  Tokens whose page id is negative write no cache.
 template <typename T>
 __global__ void __launch_bounds__(256)
 latent_prepare_kernel(const float* __restrict__ proj, int ld, int q_off, int q_rank, int kv_off, int kv_rank, int kr_off,
@@ -41,7 +41,7 @@ latent_prepare_kernel(const float* __restrict__ proj, int ld, int q_off, int q_r
     const float rs = rsqrtf(ss / (float)q_rank + eps);
     for (int i = tid; i < q_rank; i += 256) st_f32(cq + (size_t)t * q_rank + i, (row[q_off + i] * rs) * q_gain[i]);
   }
-  for (int i = tid; i < n_gate; i += 256) st_f32(gate + (size_t)t * ldg + i, row[g_off + i]);
+  for (int i = tid; i < (n_gate ? ldg : 0); i += 256) st_f32(gate + (size_t)t * ldg + i, i < n_gate ? row[g_off + i] : 0.f);
   if (!write_kv) return;
   const int page = block_table[(size_t)token_entry[t] * bt_stride + pos / page_size];
   float ss = 0.f;

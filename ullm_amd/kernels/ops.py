@@ -1144,7 +1144,7 @@ def latent_prepare(proj: torch.Tensor, q_off: int, q_rank: int, kv_off: int, kv_
         _check_pools(k_pool, v_pool, 1, page_size, hd, dtype)
     cq = torch.empty((T, q_rank), dtype=dtype, device=proj.device)
     ldg = -(-n_gate // 8) * 8
-    gate = torch.zeros((T, ldg), dtype=dtype, device=proj.device) if n_gate else None
+    gate = torch.empty((T, ldg), dtype=dtype, device=proj.device) if n_gate else None    # the kernel writes all ldg columns
     _check(build.load("latent").ullm_latent_prepare(
         _p(proj), _c_int(proj.stride(0)), _c_int(q_off), _c_int(q_rank), _c_int(kv_off), _c_int(kv_rank), _c_int(kr_off),
         _c_int(rot), _c_int(g_off), _c_int(n_gate), _p(q_gain), _p(kv_gain), _c_float(eps), _p(cos_sin), _c_int(table_rows),

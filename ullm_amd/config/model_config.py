@@ -578,3 +578,220 @@ class DovisunConfig:
     def loops(self) -> bool:
         """Whether a run of layers is passed at all (and so the embedding mixed in ahead of each pass)."""
         return self.loop_stop > self.loop_start
+
+
+# ----------------------------------------------------------------------------------------- Kumudra
+
+@dataclass(frozen=True)
+class Llama3RotaryScaling:
+    """Frequencies stretched by wavelength: pairs whose wavelength exceeds original/low turn ``factor`` times slower,
+    those below original/high are kept, those between are blended linearly in original/wavelength."""
+    factor: float
+    low: float
+    high: float
+    original: float
+
+
+@dataclass(frozen=True)
+class KumudraAttention:
+    """The softmax half of a parallel mixer: grouped-query attention with biases, a partial rotation, a window."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int                     # keys a query sees, itself included; 0: all
+    rot_dims: int                   # 0: no rotation
+    rot_base: float
+    rot_scaling: Optional[Llama3RotaryScaling]
+
+
+@dataclass(frozen=True)
+class KumudraTimeMix:
+    """The recurrent half of a parallel mixer: token-shifted projections, a decay per key channel, a bonus."""
+    heads: int
+    dim: int
+    rank: int                       # inner size of the decay's two-layer product where no checkpoint decides it
+
+
+@dataclass(frozen=True)
+class KumudraParallel:
+    left: KumudraAttention
+    right: KumudraTimeMix
+    left_scale: float
+    right_scale: float
+
+
+@dataclass(frozen=True)
+class KumudraGLA:
+    heads: int
+    dim: int
+    vdim: int
+    tau: float
+    rank: int
+
+
+@dataclass(frozen=True)
+class KumudraLightning:
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple                    # one per head
+
+
+@dataclass(frozen=True)
+class KumudraDense:
+    ff: int
+
+
+@dataclass(frozen=True)
+class KumudraExperts:
+    experts: int
+    top: int
+    ff: int
+    scale: float
+
+
+@dataclass(frozen=True)
+class KumudraLayer:
+    type: str                       # "parallel" | "gla" | "lightning"
+    mixer: object
+    mlp: object                     # KumudraDense | KumudraExperts | None
+
+
+KUMUDRA_DEFAULT_RANK = 16           # what random weights are drawn with; a checkpoint's tensors have the rank they have
+
+
+@dataclass(frozen=True)
+class KumudraConfig:
+    """Keys of a Kumudra config.json: layers listed one by one (a mixer of three kinds, a dense or routed feed-forward
+    or none), several copies of the residual stream that every sublayer reads a mix of and writes back into
+    (``streams``), a run of layers passed several times on the same tensors (``loop``), a multiplier on what joins the
+    stream, a scale on the embedding; layer norms without a bias; the head is the embedding table."""
+    architecture: str
+    vocab_size: int
+    hidden_size: int
+    layers: tuple                   # of KumudraLayer
+    norm_eps: float
+    embedding_scale: float
+    residual_mult: float
+    streams: int
+    loop_start: int
+    loop_stop: int
+    loop_times: int
+
+    @classmethod
+    def from_dict(cls, d: Mapping[str, Any]) -> "KumudraConfig":
+        norm, emb = d.get("norm") or {}, d.get("embedding") or {}
+        raw_layers = d.get("layers")
+        if not isinstance(raw_layers, (list, tuple)) or not raw_layers:
+            raise ConfigError("config.json: key 'layers' must be a non-empty list")
+        layers = []
+        for i, L in enumerate(raw_layers):
+            try:
+                if not isinstance(L, Mapping):
+                    raise ConfigError("a layer must be an object")
+                kind, m = _take(L, "type", str), L.get("mixer")
+                if not isinstance(m, Mapping):
+                    raise ConfigError("no 'mixer' object")
+                if kind == "parallel":
+                    mixer = KumudraParallel(left=_kumudra_attention(m.get("left")), right=_kumudra_time_mix(m.get("right")),
+                                            left_scale=_take(m, "left_scale", float, 1.0),
+                                            right_scale=_take(m, "right_scale", float, 1.0))
+                elif kind == "gla":
+                    dim = _take(m, "dim", int)
+                    mixer = KumudraGLA(heads=_take(m, "heads", int), dim=dim, vdim=_take(m, "vdim", int, dim),
+                                       tau=_take(m, "tau", float, 1.0), rank=_take(m, "rank", int, KUMUDRA_DEFAULT_RANK))
+                    if mixer.heads < 1 or dim < 1 or mixer.vdim < 1 or mixer.tau <= 0 or mixer.rank < 1:
+                        raise ConfigError("gated linear attention: sizes and 'tau' must be positive")
+                elif kind == "lightning":
+                    dim, decay = _take(m, "dim", int), m.get("decay")
+                    heads = _take(m, "heads", int)
+                    if not isinstance(decay, (list, tuple)) or len(decay) != heads:
+                        raise ConfigError(f"'decay' must list one number for each of the {heads} heads")
+                    mixer = KumudraLightning(heads=heads, dim=dim, vdim=_take(m, "vdim", int, dim),
+                                             decay=tuple(float(v) for v in decay))
+                    if heads < 1 or dim < 1 or mixer.vdim < 1:
+                        raise ConfigError("lightning attention: sizes must be positive")
+                else:
+                    raise ConfigError(f"type {kind!r}; known: ['gla', 'lightning', 'parallel']")
+                mlp = L.get("mlp")
+                if mlp is not None:
+                    if not isinstance(mlp, Mapping):
+                        raise ConfigError("'mlp' must be null or an object")
+                    mlp_kind = _take(mlp, "kind", str)
+                    if mlp_kind == "dense":
+                        mlp = KumudraDense(ff=_take(mlp, "ff", int))
+                        if mlp.ff < 1:
+                            raise ConfigError("'mlp.ff' must be positive")
+                    elif mlp_kind == "moe":
+                        router, expert = mlp.get("router") or {}, mlp.get("expert") or {}
+                        mlp = KumudraExperts(experts=_take(router, "experts", int), top=_take(router, "top", int),
+                                             ff=_take(expert, "ff", int), scale=_take(router, "scale", float, 1.0))
+                        if mlp.ff < 1 or not 1 <= mlp.top <= mlp.experts:
+                            raise ConfigError(f"top = {mlp.top} of {mlp.experts} experts of size {mlp.ff}")
+                    else:
+                        raise ConfigError(f"'mlp.kind' = {mlp_kind!r}; known: ['dense', 'moe']")
+            except ConfigError as e:
+                raise ConfigError(f"{e} (layer {i})") from None
+            layers.append(KumudraLayer(kind, mixer, mlp))
+        loop = d.get("loop") or {}
+        if not isinstance(loop, Mapping):
+            raise ConfigError("config.json: key 'loop' must be an object")
+        start, stop = _take(loop, "start", int, 0), _take(loop, "stop", int, 0)
+        cfg = cls(architecture=_take(d, "architecture", str, "Kumudra"), vocab_size=_take(d, "vocab", int),
+                  hidden_size=_take(d, "width", int), layers=tuple(layers), norm_eps=_take(norm, "eps", float),
+                  embedding_scale=_take(emb, "scale", float, 1.0), residual_mult=_take(d, "residual_mult", float, 1.0),
+                  streams=_take(d, "streams", int, 1), loop_start=start, loop_stop=stop,
+                  loop_times=_take(loop, "times", int, 1))
+        if cfg.vocab_size < 1 or cfg.hidden_size < 1 or cfg.norm_eps < 0 or cfg.streams < 1:
+            raise ConfigError("config.json: 'vocab', 'width' and 'streams' must be positive, 'norm.eps' not negative")
+        if not 0 <= start <= stop <= len(layers) or cfg.loop_times < 1:
+            raise ConfigError(f"config.json: 'loop' = layers {start} .. {stop} - 1, {cfg.loop_times} times, of {len(layers)} layers")
+        return cfg
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    def run_order(self) -> list:
+        """Layer indices in the order they run."""
+        n, a, b = len(self.layers), self.loop_start, self.loop_stop
+        if b <= a:
+            return list(range(n))
+        return list(range(a)) + list(range(a, b)) * self.loop_times + list(range(b, n))
+
+
+def _kumudra_attention(m) -> KumudraAttention:
+    if not isinstance(m, Mapping):
+        raise ConfigError("a parallel mixer needs a 'left' object")
+    dim = _take(m, "dim", int)
+    rot, mask = m.get("rot") or {}, m.get("mask") or {}
+    sc = rot.get("scaling")
+    scaling = None
+    if sc is not None:
+        if not isinstance(sc, Mapping):
+            raise ConfigError("'rot.scaling' must be an object")
+        scaling = Llama3RotaryScaling(factor=_take(sc, "factor", float), low=_take(sc, "low", float),
+                                      high=_take(sc, "high", float), original=_take(sc, "original", float))
+        if scaling.factor <= 0 or scaling.original <= 0 or scaling.low <= 0 or scaling.high <= 0:
+            raise ConfigError("'rot.scaling': factor, low, high and original must be positive")
+    a = KumudraAttention(heads=_take(m, "heads", int), kv_heads=_take(m, "kv_heads", int), dim=dim,
+                         vdim=_take(m, "vdim", int, dim), scale=_take(m, "scale", float, dim ** -0.5),
+                         window=_take(mask, "size", int, 0), rot_dims=_take(rot, "dims", int, 0),
+                         rot_base=_take(rot, "base", float, 10000.0), rot_scaling=scaling)
+    if a.heads < 1 or a.kv_heads < 1 or a.heads % a.kv_heads or dim < 1 or a.vdim < 1 or a.window < 0:
+        raise ConfigError(f"{a.heads} heads over {a.kv_heads} kv heads of sizes {dim} and {a.vdim}, window {a.window}")
+    if a.rot_dims < 0 or a.rot_dims % 2 or a.rot_dims > dim:
+        raise ConfigError(f"'rot.dims' = {a.rot_dims} must be even and at most 'dim' = {dim}")
+    return a
+
+
+def _kumudra_time_mix(m) -> KumudraTimeMix:
+    if not isinstance(m, Mapping):
+        raise ConfigError("a parallel mixer needs a 'right' object")
+    r = KumudraTimeMix(heads=_take(m, "heads", int), dim=_take(m, "dim", int),
+                       rank=_take(m, "rank", int, KUMUDRA_DEFAULT_RANK))
+    if r.heads < 1 or r.dim < 1 or r.rank < 1:
+        raise ConfigError("time mixing: 'heads', 'dim' and 'rank' must be positive")
+    return r

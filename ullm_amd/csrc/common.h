@@ -46,14 +46,15 @@ __device__ __forceinline__ float gated_unit(float g, float u, float limit, float
 }
 
 // Activations of an ungated feed-forward on a 32-bit value.  ACT_RELU2: max(x, 0)^2.  ACT_GELU_TANH:
-// 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))).  The product kernels' plain epilogues take ``act`` = kind + 1
+// 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))).  ACT_TANH: tanh(x).  The product kernels' plain epilogues take ``act`` = kind + 1
 // (0: none) and apply it on store.
-enum { ACT_RELU2 = 0, ACT_GELU_TANH = 1 };
+enum { ACT_RELU2 = 0, ACT_GELU_TANH = 1, ACT_TANH = 2 };
 __device__ __forceinline__ float activate(float x, int kind) {
   if (kind == ACT_RELU2) {
     const float r = fmaxf(x, 0.f);
     return r * r;
   }
+  if (kind == ACT_TANH) return tanhf(x);
   return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
 }
 __device__ __forceinline__ float activate_on_store(float x, int act) { return act ? activate(x, act - 1) : x; }

@@ -428,7 +428,7 @@ __global__ void activation_vec_kernel(const T* __restrict__ x, T* __restrict__ o
 
 extern "C" int ullm_activation(const void* x, void* out, long long total, int kind, int dtype, hipStream_t stream) {
   if (total <= 0) return 0;
-  if (kind != ACT_RELU2 && kind != ACT_GELU_TANH) return ULLM_ERR_UNSUPPORTED;
+  if (kind != ACT_RELU2 && kind != ACT_GELU_TANH && kind != ACT_TANH) return ULLM_ERR_UNSUPPORTED;
   if (total % 4 == 0 && !(((uintptr_t)x | (uintptr_t)out) & 15)) {
     const size_t total4 = (size_t)total / 4;
     dim3 vblock(256), vgrid((unsigned)((total4 + 255) / 256));

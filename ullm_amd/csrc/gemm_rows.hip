@@ -344,7 +344,7 @@ extern "C" int ullm_gemm_rows(const void* X, int ldx, const void* W, int ldw, co
   if (epi == ROWS_SILU && bias) return ULLM_ERR_UNSUPPORTED;
   if (row_sq && (M > 16 || sq_parts < 4 || sq_parts % 4 || ((uintptr_t)row_sq & 15))) return ULLM_ERR_UNSUPPORTED;
   if (unit_limit > 0.f && epi != ROWS_SILU) return ULLM_ERR_UNSUPPORTED;
-  if (act < 0 || act > 2 || (act && epi != ROWS_STORE)) return ULLM_ERR_UNSUPPORTED;
+  if (act < 0 || act > 3 || (act && epi != ROWS_STORE)) return ULLM_ERR_UNSUPPORTED;
   const RowSquares before{row_sq, sq_parts / 4, eps, unit_limit, unit_alpha, act};
   const int mt = rows_tiles(M);
   RowsShape s;

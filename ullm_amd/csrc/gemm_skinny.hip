@@ -558,7 +558,7 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
             k_per_wave = plan.k_per_wave;
   const NormAhead ahead{next_gain, (bf16_t*)next_x, next_sq, ld_next, (tiles + 3) / 4 * 4};
   if (unit_limit > 0.f && epi != EPI_SILU) return ULLM_ERR_UNSUPPORTED;
-  if (act < 0 || act > 2 || (act && epi != EPI_STORE)) return ULLM_ERR_UNSUPPORTED;
+  if (act < 0 || act > 3 || (act && epi != EPI_STORE)) return ULLM_ERR_UNSUPPORTED;
   const RowSquares before{row_sq, sq_parts / 4, unit_limit, unit_alpha, act};
   dim3 grid(tiles), block(64 * waves);
   float* R = (float*)C;

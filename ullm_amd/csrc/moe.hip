@@ -6,7 +6,9 @@
 //   route     logits [T, R] (R = experts with weights + identity experts) -> softmax over all R, the choice by
 //             softmax + correction, the `top` largest (ties: the lower index), weights = the chosen experts'
 //             softmax values over their sum (+ 1e-20).  Or (mode ROUTE_TOP_LOGITS) the `top` largest of logits +
-//             bias, weights = the softmax over those alone.  All 32-bit.  One wave per token.
+//             bias, weights = the softmax over those alone.  Or (mode ROUTE_SIGMOID) scores = sigmoid(logit) each on
+//             its own, the choice by score + correction, weights = the chosen scores over their sum (+ 1e-20).  The
+//             weights are multiplied by one constant.  All 32-bit.  One wave per token.
 //   sort      pairs (token, k) -> rows ("slots") grouped by expert; identity experts (index >= experts) get no
 //             slot.  Which slot inside its expert a pair gets depends on timing; no value does: every row of a
 //             product is a function of that row alone.  Also the tile list: (expert, first slot, rows <= tile_rows).
@@ -38,16 +40,24 @@ union Pack8 {
 // of score + correction, the chosen scores over their sum.  s_choice holds n_router floats, s_pick MOE_MAX_TOP.
 // mode ROUTE_TOP_LOGITS: `correction` is a bias on the logits; the `top` largest of logit + bias are chosen and
 // weighed by the softmax over the chosen ones alone.
-enum { ROUTE_SOFTMAX_ALL = 0, ROUTE_TOP_LOGITS = 1 };
+// mode ROUTE_SIGMOID: every score is the sigmoid of its own logit; choice and weights as for ROUTE_SOFTMAX_ALL.
+// Every weight is multiplied by `weight_scale`.
+enum { ROUTE_SOFTMAX_ALL = 0, ROUTE_TOP_LOGITS = 1, ROUTE_SIGMOID = 2 };
 __device__ __forceinline__ void route_from_logits(float* z, float* s_choice, float* s_pick,
                                                   const float* __restrict__ correction, int n_router, int top,
                                                   int* __restrict__ ids, float* __restrict__ weights, int lane,
-                                                  int mode) {
+                                                  int mode, float weight_scale) {
   if (mode == ROUTE_TOP_LOGITS) {
     for (int e = lane; e < n_router; e += 64) {
       const float v = z[e] + (correction ? correction[e] : 0.f);
       z[e] = v;
       s_choice[e] = v;
+    }
+  } else if (mode == ROUTE_SIGMOID) {
+    for (int e = lane; e < n_router; e += 64) {
+      const float s = 1.f / (1.f + expf(-z[e]));
+      z[e] = s;
+      s_choice[e] = s + (correction ? correction[e] : 0.f);
     }
   } else {
     float mx = -INFINITY;
@@ -104,32 +114,32 @@ __device__ __forceinline__ void route_from_logits(float* z, float* s_choice, flo
     const float mx = s_pick[0];
     float sum = 0.f;
     for (int k = 0; k < top; ++k) sum += expf(s_pick[k] - mx);
-    if (lane < top) weights[lane] = expf(s_pick[lane] - mx) / sum;
+    if (lane < top) weights[lane] = expf(s_pick[lane] - mx) / sum * weight_scale;
     return;
   }
-  if (lane < top) weights[lane] = s_pick[lane] / (total + 1e-20f);
+  if (lane < top) weights[lane] = s_pick[lane] / (total + 1e-20f) * weight_scale;
 }
 
 __global__ void __launch_bounds__(64)
 moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ correction, int n_router, int top,
-                 int* __restrict__ ids, float* __restrict__ weights, int mode) {
+                 int* __restrict__ ids, float* __restrict__ weights, int mode, float weight_scale) {
   __shared__ float s_soft[MOE_MAX_ROUTER], s_choice[MOE_MAX_ROUTER];
   __shared__ float s_pick[MOE_MAX_TOP];
   const int t = blockIdx.x, lane = threadIdx.x;
   for (int e = lane; e < n_router; e += 64) s_soft[e] = logits[(size_t)t * ld + e];
   __syncthreads();
   route_from_logits(s_soft, s_choice, s_pick, correction, n_router, top, ids + (size_t)t * top, weights + (size_t)t * top, lane,
-                    mode);
+                    mode, weight_scale);
 }
 
 extern "C" int ullm_moe_route(const float* logits, int ld, const float* correction, int T_, int n_router, int top,
-                              int* ids, float* weights, int mode, hipStream_t stream) {
+                              int* ids, float* weights, int mode, float weight_scale, hipStream_t stream) {
   if (T_ <= 0) return 0;
   if (n_router < 1 || n_router > MOE_MAX_ROUTER || top < 1 || top > MOE_MAX_TOP || top > n_router || ld < n_router)
     return ULLM_ERR_SHAPE;
-  if (mode != ROUTE_SOFTMAX_ALL && mode != ROUTE_TOP_LOGITS) return ULLM_ERR_UNSUPPORTED;
+  if (mode < ROUTE_SOFTMAX_ALL || mode > ROUTE_SIGMOID) return ULLM_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(moe_route_kernel, dim3(T_), dim3(64), 0, stream, logits, ld, correction, n_router, top, ids, weights,
-                     mode);
+                     mode, weight_scale);
   ULLM_LAUNCH_CHECK();
 }
 
@@ -141,7 +151,8 @@ extern "C" int ullm_moe_route(const float* logits, int ld, const float* correcti
 template <typename T, int TPB>
 __global__ void __launch_bounds__(TPB == 1 ? 1024 : 256)
 moe_router_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ correction,
-                  int n_tokens, int H, int n_router, int top, int* __restrict__ ids, float* __restrict__ weights, int mode) {
+                  int n_tokens, int H, int n_router, int top, int* __restrict__ ids, float* __restrict__ weights, int mode,
+                  float weight_scale) {
   extern __shared__ __attribute__((aligned(16))) float xrow[];          // [TPB][H]
   constexpr int RCAP = TPB == 1 ? MOE_MAX_ROUTER : 256;                // router outputs the variant takes
   __shared__ float z[TPB][RCAP], s_choice[TPB][RCAP];
@@ -204,13 +215,14 @@ moe_router_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ w,
   __syncthreads();
   if (wave < TPB && t0 + wave < n_tokens)
     route_from_logits(z[wave], s_choice[wave], s_pick[wave], correction, n_router, top, ids + (size_t)(t0 + wave) * top,
-                      weights + (size_t)(t0 + wave) * top, lane, mode);
+                      weights + (size_t)(t0 + wave) * top, lane, mode, weight_scale);
 }
 
 extern "C" int ullm_moe_router(const void* x, int ldx, const float* w, const float* correction, int T_, int H,
-                               int n_router, int top, int* ids, float* weights, int mode, int dtype, hipStream_t stream) {
+                               int n_router, int top, int* ids, float* weights, int mode, float weight_scale, int dtype,
+                               hipStream_t stream) {
   if (T_ <= 0) return 0;
-  if (mode != ROUTE_SOFTMAX_ALL && mode != ROUTE_TOP_LOGITS) return ULLM_ERR_UNSUPPORTED;
+  if (mode < ROUTE_SOFTMAX_ALL || mode > ROUTE_SIGMOID) return ULLM_ERR_UNSUPPORTED;
   if (n_router < 1 || n_router > MOE_MAX_ROUTER || top < 1 || top > MOE_MAX_TOP || top > n_router || H < 1 || ldx < H ||
       (size_t)H * sizeof(float) > 48 * 1024)
     return ULLM_ERR_SHAPE;
@@ -221,7 +233,7 @@ extern "C" int ullm_moe_router(const void* x, int ldx, const float* w, const flo
   // a token a block: sixteen waves, so that up to 64 router outputs are summed in one round of trips to memory
   dim3 grid(four ? (T_ + 3) / 4 : T_), block(four ? 256 : 1024);
 #define GO(TT, N) hipLaunchKernelGGL((moe_router_kernel<TT, N>), grid, block, lds, stream, (const TT*)x, ldx, w, correction, T_, H, \
-    n_router, top, ids, weights, mode)
+    n_router, top, ids, weights, mode, weight_scale)
   if (dtype == ULLM_F32) { if (four) GO(float, 4); else GO(float, 1); }
   else if (dtype == ULLM_BF16) { if (four) GO(bf16_t, 4); else GO(bf16_t, 1); }
   else return ULLM_ERR_DTYPE;

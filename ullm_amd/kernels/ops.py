@@ -225,11 +225,12 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     return out
 
 
-ACT_RELU2, ACT_GELU_TANH = 0, 1       # activations of an ungated feed-forward
+ACT_RELU2, ACT_GELU_TANH, ACT_TANH = 0, 1, 2       # activations behind a product
 
 
 def activation(x: torch.Tensor, kind: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """act(x) element by element, computed in 32-bit: ACT_RELU2 max(x, 0)^2, ACT_GELU_TANH the tanh form of GELU."""
+    """act(x) element by element, computed in 32-bit: ACT_RELU2 max(x, 0)^2, ACT_GELU_TANH the tanh form of GELU,
+    ACT_TANH tanh."""
     _need(x.is_contiguous(), "activation takes a contiguous tensor")
     if out is None:
         out = torch.empty_like(x)
@@ -525,6 +526,162 @@ def gated_group_norm(y: torch.Tensor, proj: torch.Tensor, z_off: int, gain: torc
     _check(build.load("recurrent").ullm_gated_group_norm(
         _p(y), _p(proj), _c_int(proj.stride(0)), _c_int(z_off), _p(gain), _c_float(eps), _p(out), _c_int(T), _c_int(width),
         _c_int(parts), _c_int(_dt(out)), _stream()), "gated_group_norm")
+    return out
+
+
+# ---------------------------------------------------------------------------------- several copies of the stream
+
+STREAMS_MAX = 8          # the most copies of the residual stream the kernels take
+
+
+def streams_spread(x: torch.Tensor, copies: int) -> torch.Tensor:
+    """float32 [copies, T, H] whose every slice is ``x`` (float32 [T, H])."""
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "x must be contiguous float32 [T, H]")
+    _need(1 <= copies <= STREAMS_MAX, f"{copies} copies of the stream: 1 to {STREAMS_MAX}")
+    out = torch.empty((copies,) + tuple(x.shape), dtype=torch.float32, device=x.device)
+    _check(build.load("streams").ullm_streams_spread(_p(x), _p(out), ctypes.c_longlong(x.numel()), _c_int(copies), _stream()),
+           "streams_spread")
+    return out
+
+
+def streams_step(streams: torch.Tensor, branch: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None,
+                 out_w: Optional[torch.Tensor] = None, mult: float = 1.0, in_w: Optional[torch.Tensor] = None,
+                 gain: Optional[torch.Tensor] = None, eps: float = 0.0, kind: int = NORM_RMS,
+                 out_dtype: Optional[torch.dtype] = None, rows: Optional[torch.Tensor] = None,
+                 second: Optional[torch.Tensor] = None, a: float = 1.0, b: float = 1.0) -> Optional[torch.Tensor]:
+    """What lies between two sublayers of a model that keeps ``streams`` (float32 [S, T, H]) copies of its residual
+    stream.  With ``branch`` ([T, H]; with ``second`` the branch is ``a * branch + b * second``): every copy t becomes
+    sum_s mix[s, t] * copy_s + mult * out_w[t] * branch, all from the old copies (``mix`` float32 [S, S] indexed
+    [from, to], ``out_w`` float32 [S]); written back in place unless ``rows``.  With ``gain``: returns the norm
+    (``kind``: NORM_RMS or NORM_LAYER, the layer norm without a bias) of sum_s in_w[s] * copy_s times ``gain`` in
+    ``out_dtype``, for all tokens or the ones ``rows`` (int32) lists.  Everything is computed in 32-bit."""
+    _need(streams.dtype == torch.float32 and streams.dim() == 3 and streams.is_contiguous(), "streams must be contiguous float32 [S, T, H]")
+    S, T, H = streams.shape
+    _need(1 <= S <= STREAMS_MAX, f"{S} copies of the stream: 1 to {STREAMS_MAX}")
+    y_dt = F32
+    if branch is not None:
+        _need(branch.shape == (T, H) and branch.is_contiguous(), "the branch must be contiguous [T, H]")
+        _need(mix is not None and mix.dtype == torch.float32 and mix.shape == (S, S) and mix.is_contiguous(), "mix must be float32 [S, S]")
+        _need(out_w is not None and out_w.dtype == torch.float32 and out_w.numel() == S and out_w.is_contiguous(), "out_w must be float32 [S]")
+        y_dt = _dt(branch)
+        if second is not None:
+            _need(second.shape == (T, H) and second.is_contiguous() and second.dtype == branch.dtype, "the second branch must match the first")
+    else:
+        _need(second is None, "a second branch needs a first")
+    n = T
+    if rows is not None:
+        _i32(rows, "rows")
+        n = rows.numel()
+    out = None
+    if gain is not None:
+        _need(gain.dtype == torch.float32 and gain.numel() == H and gain.is_contiguous(), "gain must be float32 [H]")
+        _need(in_w is not None and in_w.dtype == torch.float32 and in_w.numel() == S and in_w.is_contiguous(), "in_w must be float32 [S]")
+        out = torch.empty((n, H), dtype=out_dtype or torch.float32, device=streams.device)
+    _check(build.load("streams").ullm_streams_step(
+        _p(streams), _p(branch), _p(second), _c_float(a), _c_float(b), _c_int(y_dt), _p(mix), _p(out_w), _c_float(mult),
+        _p(in_w), _p(gain), _c_float(eps), _c_int(kind), _p(out), _c_int(_dt(out) if out is not None else F32), _p(rows),
+        _c_int(n), _c_int(T), _c_int(H), _c_int(S), _stream()), "streams_step")
+    return out
+
+
+def weighted_sum(x: torch.Tensor, y: torch.Tensor, a: float, b: float) -> torch.Tensor:
+    """float32 a * x + b * y for two contiguous tensors of one shape."""
+    _need(x.shape == y.shape and x.is_contiguous() and y.is_contiguous(), "weighted_sum takes two contiguous tensors of one shape")
+    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    _check(build.load("streams").ullm_weighted_sum(_p(x), _c_int(_dt(x)), _p(y), _c_int(_dt(y)), _c_float(a), _c_float(b),
+                                                   _p(out), ctypes.c_longlong(x.numel()), _stream()), "weighted_sum")
+    return out
+
+
+# ---------------------------------------------------------------------------------- recurrences with decays
+
+DECAY_PER_HEAD, DECAY_SIGMOID_ROOT, DECAY_EXP_EXP = 0, 1, 2      # how a recurrence's decays come about
+GATE_SILU, GATE_SIGMOID = 0, 1
+DECAY_SCAN_MAX_KEYS = 256
+
+
+def _f32_rows(t: torch.Tensor, name: str, T: int, cols: int) -> None:
+    _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape == (T, cols) and t.stride(1) == 1,
+          f"{name} must be float32 [{T}, {cols}] with unit stride along its rows")
+
+
+def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, decay_kind: int,
+               state: torch.Tensor, state_off: int, q_start: torch.Tensor, entry_slot: torch.Tensor, n_entries: int,
+               heads: int, key_dim: int, value_dim: int, tau: float = 1.0, bonus: Optional[torch.Tensor] = None,
+               silu_inputs: bool = False, q_scale: float = 1.0, write_state: bool = True) -> torch.Tensor:
+    """A recurrence per head over each entry's tokens, with the head's state S [key_dim, value_dim] (float32, at
+    ``state[slot, state_off + head * key_dim * value_dim ..]``): S = diag(d) S + k v^T and o = S^T q after the
+    update, or with ``bonus`` (float32 [heads, key_dim]) o = (S + diag(bonus) k v^T)^T q before it.  ``q``, ``k``
+    (float32 [T, heads * key_dim]) and ``v`` (float32 [T, heads * value_dim]) may be column ranges of wider rows; with
+    ``silu_inputs`` they go through silu first; q is multiplied by ``q_scale``.  The decays d: ``decay`` float32
+    [heads] (DECAY_PER_HEAD: one constant a head) or raw values z float32 [T, heads * key_dim] with d =
+    sigmoid(z)^(1/tau) (DECAY_SIGMOID_ROOT) or exp(-exp(z)) (DECAY_EXP_EXP).  Returns o float32 [T, heads * value_dim]."""
+    T = q.shape[0]
+    _f32_rows(q, "q", T, heads * key_dim)
+    _f32_rows(k, "k", T, heads * key_dim)
+    _f32_rows(v, "v", T, heads * value_dim)
+    _need(1 <= key_dim <= DECAY_SCAN_MAX_KEYS, f"{key_dim} key channels a head: at most {DECAY_SCAN_MAX_KEYS}")
+    if decay_kind == DECAY_PER_HEAD:
+        _need(decay.dtype == torch.float32 and decay.numel() == heads and decay.is_contiguous(), "decay must be float32 [heads]")
+        z_ld = 0
+    else:
+        _need(decay_kind in (DECAY_SIGMOID_ROOT, DECAY_EXP_EXP), "unknown kind of decay")
+        _f32_rows(decay, "decay", T, heads * key_dim)
+        z_ld = decay.stride(0)
+    if bonus is not None:
+        _need(bonus.dtype == torch.float32 and bonus.numel() == heads * key_dim and bonus.is_contiguous(), "bonus must be float32 [heads, key_dim]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and state_off >= 0
+          and state_off + heads * key_dim * value_dim <= state.shape[1], "state must be float32 [slots, row] holding the heads' states")
+    _i32(q_start, "q_start", n_entries + 1)
+    _i32(entry_slot, "entry_slot", n_entries)
+    out = torch.empty((T, heads * value_dim), dtype=torch.float32, device=q.device)
+    ll = ctypes.c_longlong
+    _check(build.load("decay_scan").ullm_decay_scan(
+        _p(q), _c_int(q.stride(0)), _p(k), _c_int(k.stride(0)), _p(v), _c_int(v.stride(0)), _p(decay), _c_int(z_ld),
+        _c_int(decay_kind), _c_float(tau), _p(bonus), _c_int(1 if silu_inputs else 0), _c_float(q_scale),
+        _c_int(1 if bonus is not None else 0), _p(state), ll(state.stride(0)), ll(state_off), _p(q_start), _p(entry_slot),
+        _p(out), _c_int(n_entries), _c_int(heads), _c_int(key_dim), _c_int(value_dim), _c_int(1 if write_state else 0),
+        _stream()), "decay_scan")
+    return out
+
+
+def token_shift(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, state_off: int, token_entry: torch.Tensor,
+                q_start: torch.Tensor, entry_slot: torch.Tensor, n_entries: int, write_state: bool = True) -> torch.Tensor:
+    """[M, T, H] of x's dtype: slice m is x[t] + (prev(t) - x[t]) * mu[m] (``mu`` float32 [M, H]) with prev(t) the row
+    before t in its entry or, for an entry's first token, ``state[slot, state_off .. + H]`` (float32: the last row
+    of the step before); that part of the state row then takes the entry's last row."""
+    T, H = x.shape
+    _need(x.is_contiguous(), "x must be contiguous [T, H]")
+    _need(mu.dtype == torch.float32 and mu.dim() == 2 and mu.shape[1] == H and mu.is_contiguous(), "mu must be float32 [M, H]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and 0 <= state_off
+          and state_off + H <= state.shape[1], "state must be float32 [slots, row] holding a row of H values")
+    _i32(token_entry, "token_entry", T)
+    _i32(q_start, "q_start", n_entries + 1)
+    _i32(entry_slot, "entry_slot", n_entries)
+    M = mu.shape[0]
+    out = torch.empty((M, T, H), dtype=x.dtype, device=x.device)
+    ll = ctypes.c_longlong
+    _check(build.load("decay_scan").ullm_token_shift(
+        _p(x), _p(mu), _p(state), ll(state.stride(0)), ll(state_off), _p(token_entry), _p(q_start), _p(entry_slot), _p(out),
+        _c_int(T), _c_int(H), _c_int(M), _c_int(1 if write_state else 0), _c_int(_dt(x)), _stream()), "token_shift")
+    return out
+
+
+def gated_unit_norm(o: torch.Tensor, gate: torch.Tensor, gain: torch.Tensor, eps: float, parts: int, gate_kind: int,
+                    out_dtype: torch.dtype) -> torch.Tensor:
+    """Rows ``o`` (float32 [T, width]) cut into ``parts`` equal parts, each divided by its root mean square (eps inside
+    the root), times ``gain`` (float32; as long as a part, shared by the parts, or as long as the row) and times
+    silu or sigmoid (``gate_kind``) of ``gate`` (float32 [T, width], may be a column range of wider rows)."""
+    T, width = o.shape
+    _need(o.dtype == torch.float32 and o.is_contiguous(), "o must be contiguous float32")
+    _f32_rows(gate, "gate", T, width)
+    _need(parts >= 1 and width % parts == 0, f"{width} values do not cut into {parts} equal parts")
+    _need(gain.dtype == torch.float32 and gain.is_contiguous() and gain.numel() in (width // parts, width),
+          "gain must be float32, as long as a part or as the row")
+    out = torch.empty((T, width), dtype=out_dtype, device=o.device)
+    _check(build.load("decay_scan").ullm_gated_unit_norm(
+        _p(o), _p(gate), _c_int(gate.stride(0)), _p(gain), _c_int(gain.numel()), _c_float(eps), _c_int(gate_kind), _p(out),
+        _c_int(T), _c_int(width), _c_int(parts), _c_int(_dt(out)), _stream()), "gated_unit_norm")
     return out
 
 
@@ -1216,14 +1373,17 @@ MOE_MAX_ROUTER, MOE_MAX_TOP = 1024, 32
 MOE_TILE_ROWS = (16, 32, 64, 128)     # grouped rows a block of the matrix-core expert products takes
 
 
-ROUTE_SOFTMAX_ALL, ROUTE_TOP_LOGITS = 0, 1      # how a router turns logits into experts and weights
+ROUTE_SOFTMAX_ALL, ROUTE_TOP_LOGITS, ROUTE_SIGMOID = 0, 1, 2      # how a router turns logits into experts and weights
 
 
-def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, mode: int = ROUTE_SOFTMAX_ALL):
+def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, mode: int = ROUTE_SOFTMAX_ALL,
+              weight_scale: float = 1.0):
     """(ids int32 [T, top], weights float32 [T, top]) from router logits float32 [T, R]: the softmax over all R, the
     ``top`` largest of softmax + ``correction`` (float32 [R] or None; ties go to the lower index), and as weights the
     chosen outputs' softmax values over their sum (+ 1e-20).  With ``mode`` ROUTE_TOP_LOGITS: the ``top`` largest of
-    logits + ``correction`` (a bias on the logits), weighed by the softmax over those alone."""
+    logits + ``correction`` (a bias on the logits), weighed by the softmax over those alone.  With ROUTE_SIGMOID the
+    scores are the sigmoids of the logits, each on its own; choice and weights as with the softmax.  Every weight is
+    multiplied by ``weight_scale``."""
     T, R = logits.shape
     _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "router logits must be float32 [T, R]")
     _need(1 <= top <= min(R, MOE_MAX_TOP) and R <= MOE_MAX_ROUTER, f"top {top} of {R} router outputs: at most "
@@ -1234,7 +1394,8 @@ def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int
     ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
     _check(build.load("moe").ullm_moe_route(_p(logits), _c_int(logits.stride(0)), _p(correction), _c_int(T), _c_int(R),
-                                            _c_int(top), _p(ids), _p(weights), _c_int(mode), _stream()), "moe_route")
+                                            _c_int(top), _p(ids), _p(weights), _c_int(mode), _c_float(weight_scale),
+                                            _stream()), "moe_route")
     return ids, weights
 
 
@@ -1242,7 +1403,7 @@ MOE_ROUTER_MAX_WIDTH = 12288      # widest row the fused router kernel keeps in 
 
 
 def moe_router(x: torch.Tensor, w_router: torch.Tensor, correction: Optional[torch.Tensor], top: int,
-               mode: int = ROUTE_SOFTMAX_ALL):
+               mode: int = ROUTE_SOFTMAX_ALL, weight_scale: float = 1.0):
     """:func:`moe_route` of the 32-bit product of ``x`` [T, H] with ``w_router`` (float32 [R, H]), in one kernel: every
     router output is summed along the row in an order that depends on nothing but the row."""
     T, H = x.shape
@@ -1258,7 +1419,8 @@ def moe_router(x: torch.Tensor, w_router: torch.Tensor, correction: Optional[tor
     ids = torch.empty((T, top), dtype=torch.int32, device=x.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=x.device)
     _check(build.load("moe").ullm_moe_router(_p(x), _c_int(x.stride(0)), _p(w_router), _p(correction), _c_int(T), _c_int(H),
-                                             _c_int(R), _c_int(top), _p(ids), _p(weights), _c_int(mode), _c_int(_dt(x)),
+                                             _c_int(R), _c_int(top), _p(ids), _p(weights), _c_int(mode), _c_float(weight_scale),
+                                             _c_int(_dt(x)),
                                              _stream()), "moe_router")
     return ids, weights
 

@@ -16,6 +16,7 @@ from ..cache.manager import CacheGroupSpec
 from ..kernels import ops
 from ..parts import (Block, KVNeed, LayerCache, Norm, Part, PartEnv, StateNeed, StepContext, WeightDecl,
                      build_part, cache_needs_of, walk)
+from ..parts.block import join_streams
 from ..parts.linear import linear
 
 
@@ -47,6 +48,9 @@ class ModelPlan:
     head_bias: Optional[str] = None          # tensor name of a bias [vocab] on the logits, float32
     logit_softcap: float = 0.0               # > 0: logits = cap * tanh(logits / cap)
     logit_scale: float = 1.0                 # the logits are multiplied by this
+    # > 0: the residual stream is kept in this many copies (float32 [streams, T, hidden]), all equal to the embedding
+    # output at the start; the layers' blocks read and write them, and the last norm is applied to their sum
+    streams: int = 0
     # An "embedding" part that makes the stream's first rows (several tables, state of its own); it then owns the
     # token table and ``embedding_weight`` only names it (for a tied head).  None: the plain scaled row gather.
     embedder: Optional[Choice] = None
@@ -160,6 +164,8 @@ class Model:
         else:
             residual = ops.embedding(ctx.token_ids, self.embedding, scale=self.plan.embedding_scale)
         pending = None
+        if self.plan.streams > 0:
+            residual = ops.streams_spread(residual, self.plan.streams)
         if self._keeps_embedding:
             ctx.embedded = residual.clone()      # the stream's rows are written in place from here on
         for idx, (layer, cache_id) in enumerate(self.run_order):
@@ -177,7 +183,10 @@ class Model:
                 residual, pending = block.forward(residual, pending, ctx, cache)
         if logit_rows is None or logit_rows.numel() == 0:
             return None
-        x = self.final_norm.add_norm(pending, residual, rows=logit_rows, out_dtype=ctx.dtype)
+        if self.plan.streams > 0:
+            x = join_streams(residual, pending, self.final_norm, logit_rows, ctx.dtype)
+        else:
+            x = self.final_norm.add_norm(pending, residual, rows=logit_rows, out_dtype=ctx.dtype)
         logits = linear(x, self.head, self.head_bias, out_dtype=torch.float32)
         if self.plan.logit_scale != 1.0:
             ops.scale_(logits, self.plan.logit_scale)

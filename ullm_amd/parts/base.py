@@ -35,6 +35,8 @@ class WeightDecl:
     # loader accepts any size there and the part reads it off the tensor; ``shape`` holds the size that random
     # weights are drawn with.
     free_dims: Tuple[int, ...] = ()
+    # A tensor that a checkpoint may leave out: it is then filled with this value.
+    default: Optional[float] = None
 
     def fits(self, shape) -> bool:
         shape = tuple(shape)
@@ -320,6 +322,20 @@ class NormedBranch:
     branch: torch.Tensor          # [T, hidden] in the compute dtype or float32
     post: Optional["Norm"]
     mult: float = 1.0
+
+
+@dataclass
+class StreamsBranch:
+    """A sublayer's output of a model that keeps several copies of its residual stream, not yet written back:
+    every copy t becomes sum_s mix[s, t] * copy_s + mult * out_w[t] * branch, where the branch is ``branch`` or, with
+    ``second``, ``a * branch + b * second``.  Whoever norms the streams next settles it in the same kernel."""
+    branch: torch.Tensor          # [T, hidden]
+    mix: torch.Tensor             # float32 [S, S], indexed [from, to]
+    out_w: torch.Tensor           # float32 [S]
+    mult: float = 1.0
+    second: Optional[torch.Tensor] = None
+    a: float = 1.0
+    b: float = 1.0
 
 
 class Norm(Part):

@@ -12,7 +12,8 @@ from typing import Optional
 import torch
 
 from ..kernels import ops
-from .base import Block, FeedForward, LayerCache, Mixer, Norm, NormedBranch, PendingNorm, StepContext, register_part
+from .base import (Block, FeedForward, LayerCache, Mixer, Norm, NormedBranch, PartEnv, PendingNorm, StepContext, StreamsBranch,
+                   WeightDecl, register_part)
 
 
 @register_part("block", "prenorm")
@@ -183,3 +184,105 @@ class MixInEmbedding(Block):
             branch = _one_branch(pending)
         both = ops.stream_pair(branch, mult, residual, ctx.embedded, ctx.dtype)
         return linear(both, self.w, out_dtype=torch.float32), None
+
+
+@register_part("block", "hyper_prenorm")
+class HyperPreNormBlock(Block):
+    """A pre-norm block of a model that keeps ``streams`` copies x_1 .. x_S of its residual stream (float32
+    [S, T, hidden], all equal to the embedding output at the start; the model sums them at the end).  Sublayer q
+    (the mixer, then the feed-forward if there is one) reads u = sum_s in_q[s] x_s, computes y = sublayer(norm_q(u)),
+    and then every copy at once, from the old ones, becomes x_t <- sum_s mix_q[s, t] x_s + mult * out_q[t] * y.
+    Per sublayer three small tensors: ``in`` [S], ``out`` [S], ``mix`` [S, S] (indexed [from, to]), under
+    ``<prefix>.<names[0]>`` and ``<prefix>.<names[1]>``.  With one copy and no such tensors in the checkpoint they are
+    ones: the plain pre-norm block with a multiplier.
+
+    The write-back of a sublayer and the read and norm of the next are one kernel (``ops.streams_step``): what a
+    sublayer returns travels on as a :class:`StreamsBranch` and is settled by whoever norms the streams next, the
+    next block of this kind or the model's last norm."""
+
+    def __init__(self, hidden_size: int, streams: int, mixer_norm: Norm, mixer: Mixer, prefix: str, mult: float = 1.0,
+                 ffn_norm: Optional[Norm] = None, ffn: Optional[FeedForward] = None, names=("hc1", "hc2")):
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward comes with its norm, or not at all")
+        if not 1 <= streams <= ops.STREAMS_MAX:
+            raise ValueError(f"{streams} copies of the stream: 1 to {ops.STREAMS_MAX}")
+        for norm in (mixer_norm, ffn_norm):
+            if norm is not None and type(norm).kernel_form is Norm.kernel_form:
+                raise TypeError(f"{type(norm).__name__} has no kernel form: it cannot norm a mix of streams")
+        self.hidden_size, self.streams, self.mult, self.prefix, self.names = hidden_size, int(streams), float(mult), prefix, tuple(names)
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+        self.coeffs = []                                  # per sublayer (in, out, mix)
+
+    def children(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def entry_norm(self):
+        return self.mixer_norm
+
+    def _sublayers(self):
+        return self.names[:1] if self.ffn is None else self.names[:2]
+
+    def weights(self):
+        S = self.streams
+        fill = 1.0 if S == 1 else None                    # one copy: a checkpoint may leave the coefficients out
+        out = []
+        for name in self._sublayers():
+            p = f"{self.prefix}.{name}"
+            out += [WeightDecl(f"{p}.in", (S,), init="gain", keep_fp32=True, default=fill),
+                    WeightDecl(f"{p}.out", (S,), init="gain", keep_fp32=True, default=fill),
+                    WeightDecl(f"{p}.mix", (S, S), init="gain", keep_fp32=True, default=fill)]
+        return out
+
+    def bind(self, tensors, env: PartEnv) -> None:
+        self.coeffs = [tuple(tensors[f"{self.prefix}.{name}.{k}"].contiguous() for k in ("in", "out", "mix"))
+                       for name in self._sublayers()]
+
+    def _read(self, streams, pending, norm: Norm, in_w, ctx: StepContext):
+        """Settle what is pending and return the norm of the mix the next sublayer reads."""
+        gain, eps, kind = norm.kernel_form()
+        if pending is None or isinstance(pending, PendingNorm):
+            return ops.streams_step(streams, in_w=in_w, gain=gain, eps=eps, kind=kind, out_dtype=ctx.dtype)
+        if not isinstance(pending, StreamsBranch):
+            raise TypeError("a block over several streams takes what a block of its kind left pending")
+        return ops.streams_step(streams, pending.branch, pending.mix, pending.out_w, pending.mult, in_w, gain, eps, kind,
+                                ctx.dtype, second=pending.second, a=pending.a, b=pending.b)
+
+    def _branch(self, y, coeffs) -> "StreamsBranch":
+        _, out_w, mix = coeffs
+        if isinstance(y, tuple):                          # two weighted branches, added where the streams are written
+            first, a, second, b = y
+            if first.dtype == second.dtype:
+                return StreamsBranch(first, mix, out_w, self.mult, second, a, b)
+            y = ops.weighted_sum(first, second, a, b)
+        return StreamsBranch(_one_branch(y), mix, out_w, self.mult)
+
+    def forward(self, residual, pending, ctx: StepContext, cache: LayerCache):
+        if residual.dim() != 3 or residual.shape[0] != self.streams:
+            raise RuntimeError(f"{self.prefix}: the model does not carry {self.streams} copies of its stream")
+        x = self._read(residual, pending, self.mixer_norm, self.coeffs[0][0], ctx)
+        if hasattr(self.mixer, "forward_pair"):
+            y = self.mixer.forward_pair(x, ctx, cache)
+        else:
+            y = self.mixer.forward(x, ctx, cache)
+        pending = self._branch(y, self.coeffs[0])
+        if self.ffn is None:
+            return residual, pending
+        x = self._read(residual, pending, self.ffn_norm, self.coeffs[1][0], ctx)
+        return residual, self._branch(self.ffn.forward(x, ctx), self.coeffs[1])
+
+
+def join_streams(streams, pending, norm: Norm, rows, out_dtype):
+    """The last norm of a model over several copies of its stream: what is pending is settled, the copies are added
+    and the sum is normed, for the tokens ``rows`` lists only (nothing is written back)."""
+    form = norm.kernel_form()
+    if form is None:
+        raise TypeError(f"{type(norm).__name__} has no kernel form: it cannot norm a sum of streams")
+    gain, eps, kind = form
+    ones = torch.ones((streams.shape[0],), dtype=torch.float32, device=streams.device)
+    if isinstance(pending, StreamsBranch):
+        return ops.streams_step(streams, pending.branch, pending.mix, pending.out_w, pending.mult, ones, gain, eps, kind,
+                                out_dtype, rows=rows, second=pending.second, a=pending.a, b=pending.b)
+    return ops.streams_step(streams, in_w=ones, gain=gain, eps=eps, kind=kind, out_dtype=out_dtype, rows=rows)

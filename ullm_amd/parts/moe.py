@@ -9,7 +9,9 @@ output (``correction``), the weights by the chosen outputs' scores alone, divide
 A shared expert of the same form (sizes and limit of its own) may run for every token and is added.
 Two more forms, each a parameter: ``routing="top_logits"`` picks the ``top`` largest of logits + a learned bias per
 output (the ``correction`` tensor, then a bias on the logits) and weighs them by the softmax over the picked ones
-alone; ``limit=None`` makes every expert the plain gated unit ``silu(g) * u``.
+alone; ``routing="sigmoid"`` scores every output by the sigmoid of its own logit, chooses by score + correction and
+weighs by the chosen scores over their sum (+ 1e-20); ``weight_scale`` multiplies every weight; ``limit=None`` makes
+every expert the plain gated unit ``silu(g) * u``.
 
 The experts' matrices are stacked ([experts, 2 ff, hidden] with gate rows, then up rows, per expert, and
 [experts, hidden, ff]); the loader puts the checkpoint's per-expert tensors into their rows.  A step groups
@@ -48,10 +50,11 @@ class RoutedExperts(FeedForward):
     def __init__(self, hidden_size: int, experts: int, intermediate_size: int, top: int, limit: Optional[float],
                  prefix: str, identity: int = 0, alpha: float = 1.702, correction: bool = True,
                  shared_size: int = 0, shared_limit: Optional[float] = None, names: Optional[Dict[str, str]] = None,
-                 routing: str = "softmax_all"):
-        if routing not in ("softmax_all", "top_logits"):
-            raise ValueError(f"routing={routing!r}: 'softmax_all' or 'top_logits'")
-        self.mode = ops.ROUTE_TOP_LOGITS if routing == "top_logits" else ops.ROUTE_SOFTMAX_ALL
+                 routing: str = "softmax_all", weight_scale: float = 1.0):
+        modes = {"softmax_all": ops.ROUTE_SOFTMAX_ALL, "top_logits": ops.ROUTE_TOP_LOGITS, "sigmoid": ops.ROUTE_SIGMOID}
+        if routing not in modes:
+            raise ValueError(f"routing={routing!r}: one of {sorted(modes)}")
+        self.mode, self.weight_scale = modes[routing], float(weight_scale)
         limit = 0.0 if limit is None else limit            # the kernels read a limit of 0 as the plain unit
         if experts < 0 or identity < 0 or experts + identity < 1:
             raise ValueError(f"{experts} experts and {identity} identity experts: a router needs at least one output")
@@ -106,9 +109,9 @@ class RoutedExperts(FeedForward):
     def route(self, x: torch.Tensor):
         """(ids int32 [T, top], weights float32 [T, top]) of the rows of x."""
         if self.hidden_size <= ops.MOE_ROUTER_MAX_WIDTH:
-            return ops.moe_router(x, self.w_router, self.correction, self.top, self.mode)     # the product and the routing in one
+            return ops.moe_router(x, self.w_router, self.correction, self.top, self.mode, self.weight_scale)     # the product and the routing in one
         logits = ops.gemm_simple(x, self.w_router, out_dtype=torch.float32)       # 32-bit sums in a fixed order
-        return ops.moe_route(logits, self.correction, self.top, self.mode)
+        return ops.moe_route(logits, self.correction, self.top, self.mode, self.weight_scale)
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         return self.forward_onto(x, ctx, None, None)

@@ -32,7 +32,12 @@ class Rotary(PositionEncoding):
     d(t) = rotary_dim * ln(original / (2 pi t)) / (2 ln theta), the pair index at which a pair turns t times over
     ``original`` positions, lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)), rotary_dim - 1) and
     ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns at f_i / factor * ramp_i + f_i * (1 - ramp_i),
-    and every cosine and sine is multiplied by 0.1 ln(factor) + 1."""
+    and every cosine and sine is multiplied by 0.1 ln(factor) + 1.
+
+    ``scaling`` = ("by_wavelength", factor, low, high, original) is another stretch: with l = 2 pi / f_i the pair's
+    wavelength, pairs with l < original / high keep f_i, pairs with l > original / low turn at f_i / factor, and
+    those between, with s = (original / l - low) / (high - low), at (1 - s) f_i / factor + s f_i; cosines and sines
+    keep their size."""
 
     def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None,
                  pairing: str = "half", max_positions: Optional[int] = None, scaling: Optional[tuple] = None):
@@ -45,9 +50,15 @@ class Rotary(PositionEncoding):
             raise ValueError(f"unknown rotary pairing {pairing!r}")
         self.style = 1 if pairing == "half" else 2
         self.max_positions = max_positions
-        self.scaling = None if scaling is None else tuple(float(v) for v in scaling)
-        if self.scaling is not None and (len(self.scaling) != 4 or min(self.scaling) <= 0):
-            raise ValueError(f"scaling={scaling!r}: (factor, original, fast, slow), all positive")
+        self.scaling = None
+        if scaling is not None and scaling[0] == "by_wavelength":
+            self.scaling = ("by_wavelength",) + tuple(float(v) for v in scaling[1:])
+            if len(self.scaling) != 5 or min(self.scaling[1:]) <= 0 or self.scaling[2] == self.scaling[3]:
+                raise ValueError(f"scaling={scaling!r}: ('by_wavelength', factor, low, high, original), all positive, low != high")
+        elif scaling is not None:
+            self.scaling = tuple(float(v) for v in scaling)
+            if len(self.scaling) != 4 or min(self.scaling) <= 0:
+                raise ValueError(f"scaling={scaling!r}: (factor, original, fast, slow), all positive")
         self.table: Optional[torch.Tensor] = None
 
     @staticmethod
@@ -56,6 +67,16 @@ class Rotary(PositionEncoding):
             inv_freq = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
             angles = torch.arange(rows, dtype=torch.float32)[:, None] * inv_freq[None, :]
             return torch.cat((angles.cos(), angles.sin()), dim=-1).contiguous()
+        if scaling[0] == "by_wavelength":
+            _, factor, low, high, original = scaling
+            i = torch.arange(rotary_dim // 2, dtype=torch.float64)
+            freq = torch.pow(torch.tensor(float(theta), dtype=torch.float64), -2.0 * i / rotary_dim)
+            wavelength = 2 * math.pi / freq
+            blend = ((original / wavelength - low) / (high - low)).clamp(0.0, 1.0)
+            mixed = (1.0 - blend) * freq / factor + blend * freq
+            freq = torch.where(wavelength < original / high, freq, torch.where(wavelength > original / low, freq / factor, mixed))
+            angles = torch.arange(rows, dtype=torch.float64)[:, None] * freq[None, :]
+            return torch.cat((angles.cos(), angles.sin()), dim=-1).to(torch.float32).contiguous()
         # stretched frequencies: built in 64-bit, so that the 32-bit table is the rounding of the exact angles' values
         factor, original, fast, slow = scaling
         i = torch.arange(rotary_dim // 2, dtype=torch.float64)

@@ -105,6 +105,8 @@ def check_against(decls: List[WeightDecl], index) -> None:
             continue
         if d.merged_into is not None and d.merged_into in index:
             continue
+        if d.default is not None and d.merged_into is None:
+            continue
         missing.append(f"  {name}  expected shape {list(d.shape)}")
     unexpected = []
     for n in sorted(index):
@@ -180,5 +182,10 @@ def load_weights(model, model_dir: str, env: PartEnv) -> None:
                                                             device=env.device)
                     buf[what.row_offset:what.row_offset + what.shape[0]].copy_(t)     # widens or narrows on the way
     for d in aliases:
+        if d.alias_of is None and d.default is not None:
+            # a tensor the checkpoint may leave out: filled with its declared value
+            tensors[d.name] = torch.full(d.shape, d.default, dtype=torch.float32 if d.keep_fp32 else env.dtype,
+                                         device=env.device)
+            continue
         tensors[d.name] = tensors[d.alias_of]          # tied: the same storage, no copy
     model.bind(tensors, env)

@@ -327,3 +327,13 @@ def random_weights(cfg, seed, std=None):
             t = r * (std if std is not None else 1.2 / math.sqrt(shape[-1]))
         out[name] = t.to(torch.bfloat16)
     return out
+
+
+def greedy_generate(w, cfg, prompt, n):
+    """The n tokens that follow ``prompt`` when the largest logit is taken every time (the lowest index on a tie)."""
+    toks, out = list(prompt), []
+    for _ in range(n):
+        nxt = int(torch.argmax(forward(w, cfg, toks)[-1]))
+        toks.append(nxt)
+        out.append(nxt)
+    return out

@@ -1,0 +1,644 @@
+"""Kumudra in the framework against the plain implementation (``plain_kumudra``, 64-bit): each mechanism's kernels
+alone and as one-layer models; the stream after every layer run; whole prompts; a prompt and then token by token, also
+from the very first token; portions down to two tokens; unequal requests in one batch against each alone, in a pool and
+slots that are used again; long decoding while windows pass and pages return; scores scaled so that single keys just
+inside a window decide a row; state that carries a token hundreds of steps; sizes that differ wherever they can, also
+values that make things equal or one; many requests in one captured step; greedy generation through the entry point.
+In 32-bit to rounding; in bfloat16, where a rounded router input may choose another expert at a close call, most rows to
+rounding and every clear row within a bound that a lost key, a stale slot or a state one token off exceeds."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+from safetensors.torch import save_file
+
+import plain_kumudra as plain
+from gpu_util import DEV
+
+pytestmark = pytest.mark.gpu
+
+REL = {"float32": 2e-5, "bfloat16": 3e-2}
+
+
+def gla(heads, dim, vdim, tau, mlp=None, rank=4):
+    return dict(type="gla", mixer=dict(heads=heads, dim=dim, vdim=vdim, tau=tau, rank=rank), mlp=mlp)
+
+
+def light(heads, dim, vdim, decay, mlp=None):
+    return dict(type="lightning", mixer=dict(heads=heads, dim=dim, vdim=vdim, decay=list(decay)), mlp=mlp)
+
+
+def par(heads, kv, dim, vdim, scale, window=None, rot=None, scaling=None, base=10000.0, right=(2, 8), scales=(0.6, 0.9), mlp=None, rank=4):
+    left = dict(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, scale=scale)
+    if window:
+        left["mask"] = dict(size=window)
+    if rot:
+        left["rot"] = dict(base=base, dims=rot)
+        if scaling:
+            left["rot"]["scaling"] = dict(factor=scaling[0], low=scaling[1], high=scaling[2], original=scaling[3])
+    return dict(type="parallel", mlp=mlp, mixer=dict(left=left, right=dict(heads=right[0], dim=right[1], rank=rank),
+                                                     left_scale=scales[0], right_scale=scales[1]))
+
+
+def dense(ff):
+    return dict(kind="dense", ff=ff)
+
+
+def moe(experts, top, ff, scale=1.0):
+    return dict(kind="moe", router=dict(experts=experts, top=top, scale=scale), expert=dict(ff=ff))
+
+
+def config(width, vocab, layers, streams=2, loop=None, eps=1e-5, scale=None, mult=None):
+    c = dict(architecture="Kumudra", vocab=vocab, width=width, norm=dict(eps=eps), layers=layers, streams=streams)
+    if loop:
+        c["loop"] = dict(start=loop[0], stop=loop[1], times=loop[2])
+    if scale is not None:
+        c["embedding"] = dict(scale=scale)
+    if mult is not None:
+        c["residual_mult"] = mult
+    return c
+
+
+# A: every kind of layer, the two middle ones passed twice, three copies of the stream
+CFG_A = config(48, 131, [par(6, 2, 16, 24, 0.3, window=21, rot=8, scaling=(4.0, 1.0, 4.0, 64), right=(3, 8), mlp=moe(6, 2, 20, 1.5)),
+                         gla(3, 8, 16, 8.0, mlp=dense(72)), light(2, 16, 8, (0.6, 0.995), mlp=moe(5, 3, 12, 0.8)),
+                         gla(2, 12, 12, 2.0, mlp=None)], streams=3, loop=(1, 3, 2), scale=0.7, mult=0.6)
+# B: values that make things equal or one: one copy of the stream without coefficients in the file, no loop, no scale, no
+# multiplier, as many key heads as query heads, one head, values wider and narrower than keys, no rotation, no window, an
+# unstretched rotation of the whole head, top = all experts, one expert, a layer without a feed-forward, tau 1, sizes that
+# no 16-byte access fits, decays 1 and 0
+CFG_B = config(40, 97, [par(3, 3, 6, 10, 0.5, right=(1, 6), scales=(1.0, 1.0), mlp=moe(4, 4, 9)),
+                        gla(1, 6, 10, 1.0, mlp=moe(1, 1, 14, 2.0), rank=1),
+                        light(3, 5, 7, (1.0, 0.0, 0.9), mlp=None),
+                        par(1, 1, 16, 8, 0.25, window=7, rot=16, right=(5, 4), scales=(0.2, 1.7), mlp=dense(33), rank=7)], streams=1)
+# C: head sizes of 128 and 64 in the attention, a window shorter than a page, recurrences with 64, 128 and 192 key channels,
+# four copies, the whole stack passed three times
+CFG_C = config(64, 211, [par(4, 2, 128, 64, 0.09, window=5, rot=32, scaling=(8.0, 1.0, 2.0, 32), base=100.0, right=(2, 64), mlp=moe(8, 2, 16, 1.2)),
+                         gla(2, 128, 128, 16.0, mlp=None), light(1, 192, 32, (0.97,), mlp=dense(80))], streams=4, loop=(0, 3, 3),
+               scale=1.3, mult=0.4)
+# W: attention scores of many units under a window of 33 keys, beside a weak recurrent half
+CFG_W = config(32, 64, [par(2, 1, 16, 16, 3.0, window=33, rot=8, right=(1, 4), scales=(1.0, 0.05), mlp=None)], streams=2, scale=1.0)
+# M: 8 heads of 64 value channels: 140 single tokens a step are more than a thousand (entry, head) pairs
+CFG_M = config(32, 50, [light(8, 16, 64, (0.9,) * 8, mlp=dense(24)), gla(8, 32, 64, 4.0, mlp=None)], streams=2)
+CFG_GLA = config(32, 64, [gla(2, 16, 8, 4.0, mlp=None)], streams=2)
+CFG_LIGHT = config(32, 64, [light(2, 8, 16, (0.8, 0.999), mlp=None)], streams=2)
+CFG_PAR = config(32, 64, [par(4, 2, 8, 8, 0.35, window=12, rot=4, mlp=None)], streams=2)
+CFG_DENSE = config(32, 64, [gla(1, 8, 8, 4.0, mlp=dense(40))], streams=3)
+CFG_MOE = config(32, 64, [gla(1, 8, 8, 4.0, mlp=moe(7, 3, 8, 1.5))], streams=3)
+
+MODELS = {"A": (CFG_A, 1), "B": (CFG_B, 2), "C": (CFG_C, 3), "W": (CFG_W, 4), "M": (CFG_M, 5), "gla": (CFG_GLA, 6),
+          "light": (CFG_LIGHT, 7), "par": (CFG_PAR, 8), "dense": (CFG_DENSE, 9), "moe": (CFG_MOE, 10)}
+
+
+def made_weights(name):
+    cfg, seed = MODELS[name]
+    w = plain.random_weights(cfg, seed)
+    if name == "W":
+        # queries and keys of several units a dim, so that a row's weight lies on one or two keys
+        for t in ("l0.mix.left.q", "l0.mix.left.k"):
+            w[t] = (w[t].float() * 3.0).to(torch.bfloat16)
+    return w
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    """{name: (folder, config, 64-bit weights)}; the folders hold bfloat16 tensors under the design's names."""
+    out = {}
+    for name, (cfg, _) in MODELS.items():
+        d = tmp_path_factory.mktemp(f"kumudra{name}")
+        w = made_weights(name)
+        with open(os.path.join(d, "config.json"), "w") as f:
+            json.dump(cfg, f)
+        save_file({k: v.contiguous() for k, v in w.items()}, os.path.join(d, "model.safetensors"))
+        out[name] = (str(d), cfg, {k: v.double() for k, v in w.items()})
+    return out
+
+
+_oracle_cache = {}
+
+
+def oracle(models, name, toks):
+    return oracle_and_gaps(models, name, toks)[0]
+
+
+def oracle_and_gaps(models, name, toks):
+    """(logits [T, vocab], for every row the smallest gap between the last taken and the first left choice score over
+    all routed layer runs)."""
+    key = (name, tuple(toks))
+    if key not in _oracle_cache:
+        _, cfg, w = models[name]
+        plain.MARGINS = []
+        logits = plain.forward(w, cfg, list(toks)).float().numpy()
+        gaps = np.min([m.numpy() for m in plain.MARGINS], axis=0) if plain.MARGINS else np.full(len(toks), np.inf)
+        plain.MARGINS = None
+        _oracle_cache[key] = (logits, gaps)
+    return _oracle_cache[key]
+
+
+# bfloat16 bounds (median, 85th of 100 rows, largest clear row).  A router that reads a rounded input picks another
+# expert where two choice scores lie closer than rounding moves them: such a row moves as a whole, and what it leaves in
+# the state moves the rows behind it a little.  So most rows are held to rounding, and every row whose own choices are
+# CLOSE_CALL or more apart to a bound that a lost key or a stale slot exceeds.
+BF16_BOUNDS = {"C": (4e-2, 1e-1, 0.3)}
+CLOSE_CALL = 0.02
+
+
+def close(got, want, dtype, name="", gaps=None):
+    err = np.abs(got - want).max(-1) / float(np.abs(want).max())
+    if dtype == "float32":
+        assert err.max() <= REL[dtype], f"max {err.max():.3e} at row {int(err.argmax())}"
+        return
+    mid, most, top = BF16_BOUNDS.get(name, (2e-2, 4e-2, 0.3))
+    clear = err if gaps is None else err[gaps >= CLOSE_CALL]
+    if len(err) >= 8:
+        assert np.median(err) <= mid and np.quantile(err, 0.85) <= most, \
+            f"median {np.median(err):.3e}, 85th {np.quantile(err, 0.85):.3e}"
+    elif len(clear):
+        assert np.median(clear) <= most, f"median {np.median(clear):.3e}"
+    assert not len(clear) or clear.max() <= top, f"max {clear.max():.3e} at row {int(err.argmax())}"
+
+
+def agree(models, name, toks, got, dtype, rows=None):
+    want, gaps = oracle_and_gaps(models, name, toks)
+    if rows is not None:
+        want, gaps = want[rows], gaps[rows]
+    close(got, want, dtype, name, gaps)
+
+
+def tokens(vocab, n, seed):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+@pytest.fixture(scope="module")
+def replayers(models):
+    from ullm_amd.replay import Replayer
+    made = {}
+
+    def get(name, dtype, max_tokens=512, max_requests=4, use_graphs=True):
+        key = (name, dtype, max_tokens, max_requests, use_graphs)
+        if key not in made:
+            made[key] = Replayer(models[name][0], dtype, max_tokens, 16, DEV, max_requests=max_requests, use_graphs=use_graphs)
+        rep = made[key]
+        # (a model of recurrent layers alone keeps nothing in pages)
+        assert not rep.live and (not rep.runner.cache.groups or rep.runner.cache.num_free_pages() == rep.max_tokens // 16)
+        return rep
+    return get
+
+
+def run(rep, rid, toks, cuts, end=True):
+    """Feed ``toks`` in portions of the sizes ``cuts`` (the rest one by one); logits of every position."""
+    got, at, step = [], 0, 0
+    sizes = list(cuts) + [1] * len(toks)
+    while at < len(toks):
+        n = min(sizes[step], len(toks) - at)
+        got.append(rep.step({"step": step, "entries": [{"id": rid, "tokens": toks[at:at + n], "want": list(range(n))}],
+                             "end": [rid] if end and at + n == len(toks) else []}))
+        at, step = at + n, step + 1
+    return np.concatenate(got)
+
+
+CASES = [(n, d) for n in ("A", "B", "C") for d in ("float32", "bfloat16")]
+ALONE = [(n, d) for n in ("gla", "light", "par", "dense", "moe") for d in ("float32", "bfloat16")]
+
+
+@pytest.mark.parametrize("name,dtype", CASES + ALONE)
+def test_whole_prompts(replayers, models, name, dtype):
+    rep = replayers(name, dtype)
+    for i, n in enumerate((1, 2, 15, 16, 17, 75)):
+        toks = tokens(models[name][1]["vocab"], n, 10 + i)
+        agree(models, name, toks, run(rep, "r", toks, [n]), dtype)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_the_stream_after_every_layer_run(models, name):
+    """Run by run in 32-bit: the sum of the copies once what the layer left pending is written back."""
+    from ullm_amd.engine.loading import load_model
+    from ullm_amd.engine.runner import ModelRunner, StepEntry
+    from ullm_amd.kernels import ops
+    d, cfg, w = models[name]
+    toks = tokens(cfg["vocab"], 50, 3)
+    want = []
+    plain.forward(w, cfg, toks, want)
+    _, model, env = load_model(d, "float32", DEV, context_len=64)
+    runner = ModelRunner(model, env, page_size=16, num_pages=4, max_requests=1, use_graphs=False)
+    rc = runner.cache.admit("r")
+    assert runner.cache.reserve(rc, len(toks))
+    ctx, _ = runner.build_context([StepEntry(rc, toks, [])])
+    stream = ops.streams_spread(ops.embedding(ctx.token_ids, model.embedding, scale=model.plan.embedding_scale), model.plan.streams)
+    pending, seen = None, 0
+    for block, cache_id in model.run_order:
+        stream, pending = model.blocks[block].forward(stream, pending, ctx, runner.caches.get(cache_id))
+        y = pending.a * pending.branch.double() + (pending.b * pending.second.double() if pending.second is not None else 0)
+        after = torch.einsum("sr,std->rtd", pending.mix.double(), stream.double()) + pending.mult * pending.out_w.double()[:, None, None] * y
+        after = after.sum(0).cpu()
+        assert (after - want[seen]).abs().max() <= 2e-5 * want[seen].abs().max(), seen
+        seen += 1
+    assert seen == len(want) == len(plain.run_order(cfg))
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_a_prompt_and_then_token_by_token(replayers, models, name, dtype):
+    toks = tokens(models[name][1]["vocab"], 75, 15)
+    for graphs in (True, False):
+        agree(models, name, toks, run(replayers(name, dtype, use_graphs=graphs), "r", toks, [40]), dtype)
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_token_by_token_from_the_first_token(replayers, models, name, dtype):
+    toks = tokens(models[name][1]["vocab"], 45, 16)
+    agree(models, name, toks, run(replayers(name, dtype), "r", toks, []), dtype)
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+@pytest.mark.parametrize("cuts", [(2, 2, 3, 2, 14, 2, 17, 31, 2), (1, 1, 2, 30, 3, 3, 33), (16, 16, 16, 2, 25)])
+def test_portions_of_changing_size(replayers, models, name, dtype, cuts):
+    toks = tokens(models[name][1]["vocab"], 75, 15)
+    got = run(replayers(name, dtype), "r", toks, cuts)
+    agree(models, name, toks, got, dtype)
+    if dtype == "float32":
+        # the same operations in the same order on every state element and every sum: the cutting changes no bit
+        assert np.array_equal(got, run(replayers(name, dtype), "r", toks, [75]))
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_unequal_requests_together_in_pages_and_slots_used_again(replayers, models, name, dtype):
+    """Six requests through two slots and a pool of 128 tokens: portions beside single tokens, a request left out of a
+    step, a request that starts in the slot and pages another has just given back (its state must start from zero)."""
+    rep = replayers(name, dtype, max_tokens=128, max_requests=2)
+    vocab = models[name][1]["vocab"]
+    reqs = {f"q{i}": tokens(vocab, n, 30 + i) for i, n in enumerate((50, 33, 1, 64, 20, 47))}
+    plan = [[("q0", 20), ("q1", 2)], [("q0", 1), ("q1", 31)], [("q0", 29)],          # q1 ends; q0 goes on alone
+            [("q2", 1)], [("q3", 17)], [("q3", 1)], [("q3", 2)], [("q3", 44)],        # q2 and q3 use q1's and q0's slots again
+            [("q4", 3), ("q5", 30)], [("q5", 1)], [("q4", 16), ("q5", 1)], [("q4", 1), ("q5", 15)]]
+    at = {r: 0 for r in reqs}
+    got = {r: [] for r in reqs}
+    for s, entries in enumerate(plan):
+        msg = {"step": s, "entries": [], "end": []}
+        for r, n in entries:
+            msg["entries"].append({"id": r, "tokens": reqs[r][at[r]:at[r] + n], "want": list(range(n))})
+            at[r] += n
+            if at[r] == len(reqs[r]):
+                msg["end"].append(r)
+        out, row = rep.step(msg), 0
+        for r, n in entries:
+            got[r].append(out[row:row + n])
+            row += n
+    assert at == {r: len(t) for r, t in reqs.items()}
+    for r, toks in reqs.items():
+        agree(models, name, toks, np.concatenate(got[r]), dtype)
+    rep.runner.cache.check()
+
+
+def test_many_single_tokens_in_one_captured_step(replayers, models):
+    """140 requests a step, one token each, five steps: more than a thousand (entry, head) pairs take the recurrence's
+    whole-row layout, here inside captured steps that are replayed; against the same steps run eagerly and against the
+    plain implementation."""
+    vocab = models["M"][1]["vocab"]
+    reqs = {f"m{i}": tokens(vocab, 5, 200 + i) for i in range(140)}
+    got = {}
+    for graphs in (True, False):
+        rep = replayers("M", "bfloat16", max_tokens=140 * 16, max_requests=140, use_graphs=graphs)
+        rows = {r: [] for r in reqs}
+        for step in range(5):
+            out = rep.step({"step": step, "entries": [{"id": r, "tokens": [t[step]], "want": [0]} for r, t in reqs.items()],
+                            "end": list(reqs) if step == 4 else []})
+            for i, r in enumerate(reqs):
+                rows[r].append(out[i])
+        got[graphs] = {r: np.stack(v) for r, v in rows.items()}
+    for r, toks in reqs.items():
+        assert np.abs(got[True][r] - got[False][r]).max() <= 1e-2 * np.abs(got[False][r]).max(), r
+    for r in list(reqs)[::7]:
+        agree(models, "M", reqs[r], got[True][r], "bfloat16")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_while_windows_pass_and_pages_return(replayers, models, dtype):
+    """190 tokens one by one through captured steps: the attention's window of 21 keys passes many pages, which go back
+    to the pool, the states carry on; a second request then takes the pages and the slot the first gave back."""
+    rep = replayers("A", dtype, max_tokens=192)
+    toks = tokens(models["A"][1]["vocab"], 190, 40)
+    agree(models, "A", toks, run(rep, "r", toks, [3]), dtype)
+    other = tokens(models["A"][1]["vocab"], 100, 41)
+    agree(models, "A", other, run(rep, "s", other, [60]), dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cuts", [(200,), (120,), (17, 64, 2, 31, 2, 30), (33, 33, 1, 1, 47, 47, 2, 16), (32, 1, 1, 1, 66, 34)])
+def test_keys_just_inside_the_window_decide(replayers, models, dtype, cuts):
+    """With scores of many units a softmax row lies on one or two of the window's 33 keys, in the prompt's portions and
+    for single tokens behind it: a window one key too long or too short, or a key lost at a page's border, moves the row."""
+    toks = tokens(models["W"][1]["vocab"], 200, 42)
+    want = oracle(models, "W", toks)
+    got = run(replayers("W", dtype), "r", toks, cuts)
+    if dtype == "float32":
+        close(got, want, dtype)
+    else:
+        err = np.abs(got - want).max(-1) / np.abs(want).max()
+        assert np.median(err) < 3e-2 and err.max() < 0.25, (np.median(err), err.max())
+
+
+def test_the_window_s_edge_decides_rows_in_the_peaked_model(models):
+    """The plain implementation itself: with a window one key longer or shorter several rows move by far more than
+    the bounds above (those whose weight lies on the key at the edge)."""
+    import copy
+    _, cfg, w = models["W"]
+    toks = tokens(cfg["vocab"], 200, 42)
+    base = plain.forward(w, cfg, toks)
+    for size in (32, 34):
+        c = copy.deepcopy(cfg)
+        c["layers"][0]["mixer"]["left"]["mask"]["size"] = size
+        moved = (plain.forward(w, c, toks) - base).abs().max(-1).values / base.abs().max()
+        assert int((moved > 0.05).sum()) >= 3, size
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cuts", [(300,), (1, 150, 2, 100), (290,)])
+def test_a_token_hundreds_of_steps_back_stays_in_the_state(replayers, models, dtype, cuts):
+    """The head that decays by 0.999 a token still holds the first tokens after 300 steps: the logits at the end move
+    when the first token is another one (in the plain implementation), and the framework follows."""
+    _, cfg, w = models["light"]
+    toks = tokens(cfg["vocab"], 300, 44)
+    other = [(toks[0] + 1) % cfg["vocab"]] + toks[1:]
+    base, changed = oracle(models, "light", toks), oracle(models, "light", other)
+    assert np.abs(base[-1] - changed[-1]).max() > 1e-3 * np.abs(base).max()
+    got = run(replayers("light", dtype), "r", toks, cuts)
+    agree(models, "light", toks, got, dtype)
+    if dtype == "float32":
+        got_other = run(replayers("light", dtype), "r", other, cuts)
+        moved, want_moved = got_other[-1] - got[-1], changed[-1] - base[-1]
+        assert np.abs(moved - want_moved).max() <= 0.05 * np.abs(want_moved).max()
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_greedy_generation_through_the_entry_point(models, name):
+    from ullm_amd import LLM, EngineConfig, SamplingParams
+    d, cfg, w = models[name]
+    g = torch.Generator().manual_seed(50)
+    prompts = [torch.randint(0, cfg["vocab"], (n,), generator=g).tolist() for n in (5, 19, 1, 33)]
+    for kw in (dict(), dict(max_num_batched_tokens=12, max_prefill_chunk=5, max_bs=3), dict(enforce_eager=True, disable_async_scheduling=True)):
+        args = dict(model=d, dtype="float32", max_bs=8, context_len=128, page_size=16, num_pages=24, device=DEV)
+        args.update(kw)
+        llm = LLM(EngineConfig(**args))
+        outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=10, ignore_eos=True))
+        for p, o in zip(prompts, outs):
+            assert o.token_ids == plain.greedy_generate(w, cfg, p, 10)
+        llm.engine.runner.cache.check()
+        assert llm.engine.runner.cache.num_free_pages() == 24
+        llm.shutdown()
+
+
+def test_the_trace_program_runs_the_design(models, trace_run):
+    d, cfg, _ = models["A"]
+    toks = tokens(cfg["vocab"], 40, 60)
+    want = oracle(models, "A", toks)
+    tr = trace_run(d, "float32", 128)
+    a = tr.step([("a", toks[:21], [0, 20])])
+    b = tr.step([("a", toks[21:], [18])], end=["a"])
+    tr.close()
+    close(np.concatenate((a, b)), want[[0, 20, 39]], "float32")
+
+
+def test_one_copy_of_the_stream_with_and_without_coefficients_in_the_file(models, tmp_path):
+    """A checkpoint of a model with one copy may hold the coefficients (here: not ones) or leave them out (ones)."""
+    from ullm_amd.replay import Replayer
+    d, cfg, w = models["B"]
+    assert not any(".hc" in k for k in w)
+    g = torch.Generator().manual_seed(5)
+    more = dict(made_weights("B"))
+    for i, L in enumerate(cfg["layers"]):
+        for q in (1, 2) if L["mlp"] else (1,):
+            more.update({f"l{i}.hc{q}.in": (1.0 + 0.3 * torch.randn(1, generator=g)).to(torch.bfloat16),
+                         f"l{i}.hc{q}.out": (1.0 + 0.3 * torch.randn(1, generator=g)).to(torch.bfloat16),
+                         f"l{i}.hc{q}.mix": (1.0 + 0.3 * torch.randn(1, 1, generator=g)).to(torch.bfloat16)})
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.contiguous() for k, v in more.items()}, str(tmp_path / "model.safetensors"))
+    toks = tokens(cfg["vocab"], 30, 70)
+    rep = Replayer(str(tmp_path), "float32", 64, 16, DEV, max_requests=1)
+    got = run(rep, "r", toks, [11])
+    # the plain implementation's general form on one copy
+    wide = {k: v.double() for k, v in more.items()}
+    eps, x = cfg["norm"]["eps"], wide["embed"][torch.tensor(toks)][None]
+    for i, L in enumerate(cfg["layers"]):
+        p = f"l{i}"
+        x = plain.hyper_sublayer(x, lambda u: plain.MIXERS[L["type"]](plain.layer_norm(u, wide[p + ".norm1"], eps), wide, p + ".mix", L["mixer"], eps), wide, p, 1, 1.0)
+        if L["mlp"]:
+            x = plain.hyper_sublayer(x, lambda u: plain.feed_forward(plain.layer_norm(u, wide[p + ".norm2"], eps), wide, p + ".mlp", L["mlp"]), wide, p, 2, 1.0)
+    want = (plain.layer_norm(x.sum(0), wide["final.norm"], eps) @ wide["embed"].T).float().numpy()
+    close(got, want, "float32")
+    assert np.abs(want - oracle(models, "B", toks)).max() > 1e-2 * np.abs(want).max()     # the coefficients matter
+
+
+# ------------------------------------------------------------------------------------------- kernels alone
+
+def _entries(lens, device):
+    """(token_entry, q_start, entry_slot with slots in another order) for entries of these lengths."""
+    q_start = np.concatenate(([0], np.cumsum(lens))).astype(np.int32)
+    token_entry = np.repeat(np.arange(len(lens)), lens).astype(np.int32)
+    slots = np.arange(len(lens))[::-1].astype(np.int32) + 1
+    to = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)      # noqa: E731
+    return to(token_entry), to(q_start), to(slots)
+
+
+@pytest.mark.parametrize("heads,N,P", [(1, 1, 1), (3, 6, 10), (2, 32, 64), (4, 64, 16), (2, 128, 128), (1, 200, 24), (2, 17, 33)])
+@pytest.mark.parametrize("kind", ["per_head", "sigmoid_root", "exp_exp_bonus"])
+def test_the_recurrence_alone(heads, N, P, kind):
+    """Three requests in two steps each (portions of 1 to 37 tokens, in one batch, slots in another order than the
+    entries), the state carried in rows that hold other values ahead of the heads' states."""
+    from ullm_amd.kernels import ops
+    g = torch.Generator().manual_seed(heads * 1000 + N * 10 + P)
+    lens_a, lens_b = [37, 1, 5], [2, 18, 1]
+    total = [a + b for a, b in zip(lens_a, lens_b)]
+    seqs = []
+    for n in total:
+        q, k = torch.randn(n, heads, N, generator=g) * 0.6, torch.randn(n, heads, N, generator=g) * 0.6
+        v = torch.randn(n, heads, P, generator=g)
+        z = torch.randn(n, heads, N, generator=g) * 2.0
+        seqs.append((q, k, v, z))
+    tau, bonus, dec_head = 3.0, torch.randn(heads, N, generator=g), torch.rand(heads, generator=g)
+    silu_in, q_scale = kind == "per_head", 0.5 if kind == "sigmoid_root" else 1.0
+    want = []
+    for q, k, v, z in seqs:
+        qd, kd, vd, zd = q.double(), k.double(), v.double(), z.double()
+        if silu_in:
+            qd, kd, vd = plain.silu(qd), plain.silu(kd), plain.silu(vd)
+        if kind == "per_head":
+            d = dec_head.double()[None, :, None].expand_as(qd)
+        elif kind == "sigmoid_root":
+            d = torch.sigmoid(zd).pow(1.0 / tau)
+        else:
+            d = torch.exp(-torch.exp(zd))
+        want.append(plain.decayed_state_outputs(qd * q_scale, kd, vd, d, bonus.double() if kind == "exp_exp_bonus" else None))
+    off = 7
+    state = torch.full((5, off + heads * N * P), 3.0, device=DEV)
+    state[:, off:] = 0.0
+    got = [[] for _ in seqs]
+    at = [0, 0, 0]
+    for lens in (lens_a, lens_b):
+        _, q_start, slots = _entries(lens, DEV)
+        cat = lambda i, width: torch.cat([s[i][a:a + n].reshape(n, heads * width) for s, a, n in zip(seqs, at, lens)]).to(DEV)   # noqa: E731
+        wide = torch.cat((cat(0, N), cat(1, N), cat(2, P)), dim=1).contiguous()          # column ranges of wider rows
+        q, k, v = wide[:, :heads * N], wide[:, heads * N:2 * heads * N], wide[:, 2 * heads * N:]
+        if kind == "per_head":
+            o = ops.decay_scan(q, k, v, dec_head.to(DEV), ops.DECAY_PER_HEAD, state, off, q_start, slots, 3, heads, N, P, silu_inputs=True)
+        elif kind == "sigmoid_root":
+            o = ops.decay_scan(q, k, v, cat(3, N), ops.DECAY_SIGMOID_ROOT, state, off, q_start, slots, 3, heads, N, P, tau=tau, q_scale=q_scale)
+        else:
+            o = ops.decay_scan(q, k, v, cat(3, N), ops.DECAY_EXP_EXP, state, off, q_start, slots, 3, heads, N, P, bonus=bonus.to(DEV))
+        row = 0
+        for i, n in enumerate(lens):
+            got[i].append(o[row:row + n].cpu())
+            row += n
+            at[i] += n
+    for i, w in enumerate(want):
+        g_i = torch.cat(got[i]).double().view_as(w)
+        assert (g_i - w).abs().max() <= 2e-5 * w.abs().max() + 1e-6, i
+    assert bool((state[:, :off] == 3.0).all()) and bool((state[0, off:] == 0).all()) and bool((state[4, off:] == 0).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_the_blend_with_the_previous_token(dtype):
+    from ullm_amd.kernels import ops
+    g = torch.Generator().manual_seed(3)
+    H, M = 24, 5
+    mu = torch.rand(M, H, generator=g)
+    xs = [torch.randn(n, H, generator=g).to(dtype) for n in (9, 3, 4)]
+    state = torch.zeros(5, 4 + H, device=DEV)
+    got, at = [[] for _ in xs], [0, 0, 0]
+    for lens in ([4, 1, 2], [5, 2, 2]):
+        token_entry, q_start, slots = _entries(lens, DEV)
+        x = torch.cat([s[a:a + n] for s, a, n in zip(xs, at, lens)]).to(DEV)
+        out = ops.token_shift(x, mu.to(DEV), state, 4, token_entry, q_start, slots, 3)
+        assert out.dtype == dtype and out.shape == (M, sum(lens), H)
+        row = 0
+        for i, n in enumerate(lens):
+            got[i].append(out[:, row:row + n].float().cpu())
+            row += n
+            at[i] += n
+    for i, x in enumerate(xs):
+        xd = x.double()
+        prev = torch.cat((torch.zeros(1, H, dtype=torch.float64), xd[:-1]))
+        want = xd[None] + (prev - xd)[None] * mu.double()[:, None, :]
+        assert (torch.cat(got[i], dim=1).double() - want).abs().max() <= (1e-6 if dtype == torch.float32 else 2e-2)
+    assert bool((state[:, :4] == 0).all()) and torch.equal(state[3, 4:].cpu(), xs[0][-1].float())
+
+
+@pytest.mark.parametrize("parts,shared", [(4, True), (4, False), (1, False), (3, True)])
+@pytest.mark.parametrize("gate_kind", ["silu", "sigmoid"])
+def test_the_norm_of_the_outputs_with_gain_and_gate(parts, shared, gate_kind):
+    from ullm_amd.kernels import ops
+    g = torch.Generator().manual_seed(parts)
+    T, size = 11, 10
+    width = parts * size
+    o, wide = torch.randn(T, width, generator=g) * 3, torch.randn(T, width + 6, generator=g)
+    gain = 1 + 0.3 * torch.randn(size if shared else width, generator=g)
+    gate = wide[:, 6:]
+    z = gate.double()
+    act = plain.silu(z) if gate_kind == "silu" else torch.sigmoid(z)
+    full_gain = gain.double().repeat(parts) if shared else gain.double()
+    want = plain.unit_rms(o.double().view(T, parts, size), 1e-5).reshape(T, width) * full_gain * act
+    for dtype in (torch.float32, torch.bfloat16):
+        got = ops.gated_unit_norm(o.to(DEV), wide.to(DEV)[:, 6:], gain.to(DEV), 1e-5, parts,
+                                  ops.GATE_SILU if gate_kind == "silu" else ops.GATE_SIGMOID, dtype)
+        assert got.dtype == dtype
+        assert (got.double().cpu() - want).abs().max() <= (2e-5 if dtype == torch.float32 else 2e-2) * want.abs().max()
+
+
+@pytest.mark.parametrize("S,H", [(1, 8), (2, 40), (3, 300), (4, 1024), (8, 33)])
+@pytest.mark.parametrize("kind", ["layer", "rms"])
+def test_what_lies_between_two_sublayers_over_several_copies(S, H, kind):
+    """Write-back alone, read and norm alone, both in one kernel, two weighted branches, and the last norm on chosen
+    rows without a write-back."""
+    from ullm_amd.kernels import ops
+    g = torch.Generator().manual_seed(S * 7 + H)
+    T = 9
+    xs = torch.randn(S, T, H, generator=g)
+    mix, out_w, in_w = torch.randn(S, S, generator=g), torch.randn(S, generator=g), torch.randn(S, generator=g)
+    gain = 1 + 0.2 * torch.randn(H, generator=g)
+    ya, yb = torch.randn(T, H, generator=g), torch.randn(T, H, generator=g)
+    eps, mult, a, b = 1e-5, 0.7, 0.6, -1.3
+    k = ops.NORM_LAYER if kind == "layer" else ops.NORM_RMS
+
+    def norm(u):
+        return plain.layer_norm(u, gain.double(), eps) if kind == "layer" else plain.unit_rms(u, eps) * gain.double()
+
+    def written(y):
+        return torch.einsum("sr,std->rtd", mix.double(), xs.double()) + mult * out_w.double()[:, None, None] * y[None]
+
+    dev = lambda t: t.to(DEV)      # noqa: E731
+    # read and norm alone
+    got = ops.streams_step(dev(xs).clone(), in_w=dev(in_w), gain=dev(gain), eps=eps, kind=k, out_dtype=torch.float32)
+    want = norm(torch.einsum("s,std->td", in_w.double(), xs.double()))
+    assert (got.double().cpu() - want).abs().max() <= 2e-5 * want.abs().max()
+    for dtype in (torch.float32, torch.bfloat16):
+        y1, y2 = ya.to(dtype), yb.to(dtype)
+        tol = 2e-5
+        # write-back alone
+        s = dev(xs).clone()
+        assert ops.streams_step(s, dev(y1), dev(mix), dev(out_w), mult) is None
+        new = written(y1.double())
+        assert (s.double().cpu() - new).abs().max() <= tol * new.abs().max()
+        # both, with two weighted branches
+        s = dev(xs).clone()
+        got = ops.streams_step(s, dev(y1), dev(mix), dev(out_w), mult, dev(in_w), dev(gain), eps, k, torch.float32,
+                               second=dev(y2), a=a, b=b)
+        new = written(a * y1.double() + b * y2.double())
+        want = norm(torch.einsum("s,std->td", in_w.double(), new))
+        assert (s.double().cpu() - new).abs().max() <= tol * new.abs().max()
+        assert (got.double().cpu() - want).abs().max() <= 5e-5 * want.abs().max()
+        # the last norm: chosen rows of the copies' sum, nothing written back
+        s = dev(xs).clone()
+        rows = torch.tensor([7, 0, 3], dtype=torch.int32, device=DEV)
+        got = ops.streams_step(s, dev(y1), dev(mix), dev(out_w), mult, dev(torch.ones(S)), dev(gain), eps, k, torch.float32, rows=rows)
+        want = norm(written(y1.double()).sum(0))[[7, 0, 3]]
+        assert torch.equal(s.cpu(), xs) and (got.double().cpu() - want).abs().max() <= 5e-5 * want.abs().max()
+    assert torch.equal(ops.streams_spread(dev(xs[0]).contiguous(), S).cpu(), xs[0][None].expand(S, T, H))
+    assert (ops.weighted_sum(dev(ya), dev(yb.to(torch.bfloat16)), a, b).cpu() - (a * ya + b * yb.to(torch.bfloat16).float())).abs().max() <= 1e-6
+
+
+@pytest.mark.parametrize("R,top", [(1, 1), (5, 5), (7, 3), (64, 8), (130, 2)])
+def test_sigmoid_scores_choice_with_correction_and_scaled_weights(R, top):
+    from ullm_amd.kernels import ops
+    g = torch.Generator().manual_seed(R)
+    T, H = 12, 40
+    logits = torch.randn(T, R, generator=g) * 2
+    logits[0] = 0.0                                      # a row of ties: the lower indices are taken
+    logits[1] = -40.0                                    # scores that vanish: the sum's guard
+    corr = torch.randn(R, generator=g) * 0.5
+    s = torch.sigmoid(logits.double())
+    order = torch.sort(s + corr.double(), dim=-1, descending=True, stable=True).indices[:, :top]
+    want_w = torch.gather(s, 1, order)
+    want_w = want_w / (want_w.sum(-1, keepdim=True) + 1e-20) * 2.5
+    ids, weights = ops.moe_route(logits.to(DEV), corr.to(DEV), top, ops.ROUTE_SIGMOID, 2.5)
+    assert torch.equal(ids.cpu().long(), order) and (weights.double().cpu() - want_w).abs().max() <= 1e-5
+    # the product and the routing in one kernel, from bfloat16-representable inputs
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    w = torch.randn(R, H, generator=g)
+    z = x.double() @ w.double().T
+    s = torch.sigmoid(z)
+    choice = s + corr.double()
+    vals = torch.sort(choice, dim=-1, descending=True).values
+    clear = (vals[:, :-1] - vals[:, 1:]).min(-1).values > 1e-4 if R > 1 else torch.ones(T, dtype=torch.bool)
+    order = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
+    for dtype in (torch.float32, torch.bfloat16):
+        ids, weights = ops.moe_router(x.to(DEV, dtype), w.to(DEV), corr.to(DEV), top, ops.ROUTE_SIGMOID, 2.5)
+        assert torch.equal(ids.cpu().long()[clear], order[clear])
+        want_w = torch.gather(s, 1, order)
+        want_w = want_w / (want_w.sum(-1, keepdim=True) + 1e-20) * 2.5
+        assert (weights.double().cpu() - want_w)[clear].abs().max() <= 1e-4
+
+
+def test_tanh_on_store_of_the_products():
+    from ullm_amd.kernels import ops
+    from ullm_amd.parts.linear import linear
+    g = torch.Generator().manual_seed(9)
+    for M in (1, 9, 40, 300):
+        x, w = torch.randn(M, 64, generator=g).to(torch.bfloat16), (torch.randn(16, 64, generator=g) * 0.2).to(torch.bfloat16)
+        want = torch.tanh(x.double() @ w.double().T)
+        got = linear(x.to(DEV), w.to(DEV), out_dtype=torch.float32, act=ops.ACT_TANH)
+        assert (got.double().cpu() - want).abs().max() <= 1e-5
+        got = linear(x.float().to(DEV), w.float().to(DEV), act=ops.ACT_TANH)
+        assert (got.double().cpu() - want).abs().max() <= 1e-5

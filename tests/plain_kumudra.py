@@ -218,17 +218,19 @@ def hyper_sublayer(xs, fn, w, p, q, mult):
     return torch.einsum("sr,std->rtd", w[f"{p}.hc{q}.mix"], xs) + mult * w[f"{p}.hc{q}.out"][:, None, None] * y[None]
 
 
-def forward(w, cfg, tokens, layers_out=None):
+def forward(w, cfg, tokens, layers_out=None, round_to=None):
     """Logits [T, vocab] of one sequence from its first token; ``layers_out`` receives the stream (the sum of the
-    streams) after every layer run."""
+    streams) after every layer run.  With ``round_to`` every sublayer's input is rounded to that dtype on its way
+    (what a model loses at the least when its products read such inputs)."""
+    rounded = (lambda t: t.to(round_to).to(F)) if round_to is not None else (lambda t: t)
     eps, mult = cfg["norm"]["eps"], cfg.get("residual_mult", 1.0)
     streams = cfg.get("streams", 1)
     x = w["embed"][torch.tensor(tokens)] * (cfg.get("embedding") or {}).get("scale", 1.0)
     xs = x[None].repeat(streams, 1, 1) if streams > 1 else None
     for i in run_order(cfg):
         L, p = cfg["layers"][i], f"l{i}"
-        mixer = lambda u: MIXERS[L["type"]](layer_norm(u, w[p + ".norm1"], eps), w, p + ".mix", L["mixer"], eps)   # noqa: E731
-        ff = lambda u: feed_forward(layer_norm(u, w[p + ".norm2"], eps), w, p + ".mlp", L["mlp"])                    # noqa: E731
+        mixer = lambda u: MIXERS[L["type"]](rounded(layer_norm(u, w[p + ".norm1"], eps)), w, p + ".mix", L["mixer"], eps)   # noqa: E731
+        ff = lambda u: feed_forward(rounded(layer_norm(u, w[p + ".norm2"], eps)), w, p + ".mlp", L["mlp"])                    # noqa: E731
         if streams > 1:
             xs = hyper_sublayer(xs, mixer, w, p, 1, mult)
             if L.get("mlp"):
@@ -240,7 +242,7 @@ def forward(w, cfg, tokens, layers_out=None):
                 x = x + mult * ff(x)
         if layers_out is not None:
             layers_out.append(x.clone())
-    return layer_norm(x, w["final.norm"], eps) @ w["embed"].T
+    return rounded(layer_norm(x, w["final.norm"], eps)) @ w["embed"].T
 
 
 # ----------------------------------------------------------------------------- random weights

@@ -231,7 +231,7 @@ def test_parts_are_found_by_name_and_unknown_names_fail():
     from ullm_amd.parts import build_part, registered_parts
     assert "toy_running_mean" in registered_parts("mixer") and "gqa_attention" in registered_parts("mixer")
     assert "toy_keys_only" in registered_parts("mixer")
-    assert "swiglu" in registered_parts("ffn") and registered_parts("block") == ["mix_in_embedding", "parallel", "prenorm", "sandwich", "toy_two_mixers"]
+    assert "swiglu" in registered_parts("ffn") and registered_parts("block") == ["hyper_prenorm", "mix_in_embedding", "parallel", "prenorm", "sandwich", "toy_two_mixers"]
     assert "routed_experts" in registered_parts("ffn") and "mlp" in registered_parts("ffn") and "latent_attention" in registered_parts("mixer")
     assert "mamba2" in registered_parts("mixer") and "layernorm" in registered_parts("norm")
     assert "table_sum" in registered_parts("embedding") and "log_distance_bias" in registered_parts("position")

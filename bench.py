@@ -55,11 +55,13 @@ def parse_args():
                     help="instead of the default workload: Pamopel (attention with a distance bias and head gates, a "
                          "layer on another's keys and values, a Mamba-2 layer) beside a Qwen3 stack of the same width, "
                          f"heads, feed-forward, vocabulary and depth, random weights; shapes: {sorted(DESIGN_SHAPES)}")
-    ap.add_argument("--design-model", choices=("both", "all", "pamopel", "qwen3", "ziferax", "dovisun"), default="both",
+    ap.add_argument("--design-model", choices=("both", "all", "pamopel", "qwen3", "ziferax", "dovisun", "kumudra"), default="both",
                     help="with --design: one design only (for profiles), Pamopel and Qwen3 (both), or these, Ziferax "
                          "(a stack of parallel blocks of windowed attention with sinks and a routed feed-forward) and "
                          "Dovisun (parallel blocks of unit-norm attention with a fixed sink or latent attention, dense "
-                         "or routed feed-forwards, two layers passed twice) (all)")
+                         "or routed feed-forwards, two layers passed twice) and Kumudra (two copies of the residual "
+                         "stream, gated linear attention, lightning attention and windowed attention beside time "
+                         "mixing, four layers passed twice) (all)")
     ap.add_argument("--prefill-only", type=int, default=0, metavar="T",
                     help="only time a T-token prompt and print its figures (for profiling)")
     return ap.parse_args()
@@ -189,13 +191,31 @@ def dovisun_config(shape):
                 embedding=dict(scale=float(W) ** 0.5), logit_softcap=30.0, loop=dict(start=2, stop=4, times=2))
 
 
+# Kumudra at a design shape: the same width; four layers passed twice, so eight layer runs a token as the other stacks
+# have, over two copies of the residual stream: gated linear attention (keys of half the head size) with the dense
+# feed-forward, two lightning layers and one layer of windowed attention (the other stacks' heads, a window of 1024 keys,
+# half of each head rotated) beside time mixing (heads of 64), these three with routed feed-forwards of as many columns
+# a token as the dense one (top 4 of 32 experts of a sixth of it).
+def kumudra_config(shape):
+    (W, H, G, D, F, L), _ = DESIGN_SHAPES[shape]
+    moe = dict(kind="moe", router=dict(experts=32, top=4, scale=2.5), expert=dict(ff=F // 6))
+    lightning = dict(heads=H, dim=D, vdim=D, decay=[1.0 - 2.0 ** (-5.0 - 4.0 * h / max(1, H - 1)) for h in range(H)])
+    left = dict(heads=H, kv_heads=G, dim=D, vdim=D, scale=D ** -0.5, mask=dict(size=1024),
+                rot=dict(base=500000.0, dims=D // 2, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)))
+    layers = [dict(type="gla", mixer=dict(heads=H, dim=D // 2, vdim=D, tau=16.0), mlp=dict(kind="dense", ff=F)),
+              dict(type="lightning", mixer=lightning, mlp=moe), dict(type="lightning", mixer=lightning, mlp=moe),
+              dict(type="parallel", mlp=moe, mixer=dict(left=left, right=dict(heads=W // 64, dim=64), left_scale=0.6, right_scale=0.9))]
+    return dict(architecture="Kumudra", vocab=DESIGN_VOCAB, width=W, norm=dict(eps=1e-5), layers=layers, streams=2,
+                residual_mult=0.7, embedding=dict(scale=1.0), loop=dict(start=0, stop=4, times=max(1, L // 4)))
+
+
 def design_run(args):
     """Decode at batch 1 / 8 / 64 (1024-token prompts) and one 2048-token prompt, for the designs of a shape."""
     out = {"metric": f"decode and prefill tok/s, designs beside Qwen3 at shape {args.design}, random weights",
            "unit": "tokens/s", "dtype": args.dtype, "data": "synthetic", "shape": args.design, "designs": {}}
-    configs = design_configs(args.design) + (ziferax_config(args.design), dovisun_config(args.design))
-    for label, config in zip(("pamopel", "qwen3", "ziferax", "dovisun"), configs):
-        if args.design_model not in ("both", "all", label) or (label in ("ziferax", "dovisun") and args.design_model == "both"):
+    configs = design_configs(args.design) + (ziferax_config(args.design), dovisun_config(args.design), kumudra_config(args.design))
+    for label, config in zip(("pamopel", "qwen3", "ziferax", "dovisun", "kumudra"), configs):
+        if args.design_model not in ("both", "all", label) or (label in ("ziferax", "dovisun", "kumudra") and args.design_model == "both"):
             continue
         m = Sized(label, args.dtype, 4096, eager=args.eager, config=config)
         rec = {"weights_GB": round(m.wbytes / 1e9, 3), "decode": {}}

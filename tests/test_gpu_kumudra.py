@@ -445,13 +445,15 @@ def _entries(lens, device):
 
 @pytest.mark.parametrize("heads,N,P", [(1, 1, 1), (3, 6, 10), (2, 32, 64), (4, 64, 16), (2, 128, 128), (1, 200, 24), (2, 17, 33)])
 @pytest.mark.parametrize("kind", ["per_head", "sigmoid_root", "exp_exp_bonus"])
-def test_the_recurrence_alone(heads, N, P, kind):
-    """Three requests in two steps each (portions of 1 to 37 tokens, in one batch, slots in another order than the
-    entries), the state carried in rows that hold other values ahead of the heads' states."""
+@pytest.mark.parametrize("ahead", [False, True])
+def test_the_recurrence_alone(heads, N, P, kind, ahead):
+    """Three requests in three steps each (portions of 1 to 37 tokens in one batch, then a step of single tokens; slots
+    in another order than the entries), the state carried in rows that hold other values ahead of the heads' states;
+    with the inputs' functions applied inside the recurrence or by the pass ahead of it."""
     from ullm_amd.kernels import ops
     g = torch.Generator().manual_seed(heads * 1000 + N * 10 + P)
-    lens_a, lens_b = [37, 1, 5], [2, 18, 1]
-    total = [a + b for a, b in zip(lens_a, lens_b)]
+    lens_a, lens_b, lens_c = [37, 1, 5], [2, 18, 1], [1, 1, 1]
+    total = [a + b + c for a, b, c in zip(lens_a, lens_b, lens_c)]
     seqs = []
     for n in total:
         q, k = torch.randn(n, heads, N, generator=g) * 0.6, torch.randn(n, heads, N, generator=g) * 0.6
@@ -477,17 +479,26 @@ def test_the_recurrence_alone(heads, N, P, kind):
     state[:, off:] = 0.0
     got = [[] for _ in seqs]
     at = [0, 0, 0]
-    for lens in (lens_a, lens_b):
+    for lens in (lens_a, lens_b, lens_c):
         _, q_start, slots = _entries(lens, DEV)
         cat = lambda i, width: torch.cat([s[i][a:a + n].reshape(n, heads * width) for s, a, n in zip(seqs, at, lens)]).to(DEV)   # noqa: E731
         wide = torch.cat((cat(0, N), cat(1, N), cat(2, P)), dim=1).contiguous()          # column ranges of wider rows
         q, k, v = wide[:, :heads * N], wide[:, heads * N:2 * heads * N], wide[:, 2 * heads * N:]
+        most = dict(max_len=max(lens))
         if kind == "per_head":
-            o = ops.decay_scan(q, k, v, dec_head.to(DEV), ops.DECAY_PER_HEAD, state, off, q_start, slots, 3, heads, N, P, silu_inputs=True)
-        elif kind == "sigmoid_root":
-            o = ops.decay_scan(q, k, v, cat(3, N), ops.DECAY_SIGMOID_ROOT, state, off, q_start, slots, 3, heads, N, P, tau=tau, q_scale=q_scale)
+            if ahead:
+                ops.decay_prepare(wide)
+            o = ops.decay_scan(q, k, v, dec_head.to(DEV), ops.DECAY_PER_HEAD, state, off, q_start, slots, 3, heads, N, P,
+                               silu_inputs=not ahead, **most)
         else:
-            o = ops.decay_scan(q, k, v, cat(3, N), ops.DECAY_EXP_EXP, state, off, q_start, slots, 3, heads, N, P, bonus=bonus.to(DEV))
+            z, raw = cat(3, N), ops.DECAY_SIGMOID_ROOT if kind == "sigmoid_root" else ops.DECAY_EXP_EXP
+            if ahead:
+                ops.decay_prepare(None, z, raw, tau)
+            how = ops.DECAY_READY if ahead else raw
+            if kind == "sigmoid_root":
+                o = ops.decay_scan(q, k, v, z, how, state, off, q_start, slots, 3, heads, N, P, tau=tau, q_scale=q_scale, **most)
+            else:
+                o = ops.decay_scan(q, k, v, z, how, state, off, q_start, slots, 3, heads, N, P, bonus=bonus.to(DEV), **most)
         row = 0
         for i, n in enumerate(lens):
             got[i].append(o[row:row + n].cpu())

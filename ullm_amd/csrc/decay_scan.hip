@@ -15,7 +15,8 @@
 // cut, and a token's output sums its partial sums in a fixed order.
 #include "common.h"
 
-enum { DECAY_PER_HEAD = 0, DECAY_SIGMOID_ROOT = 1, DECAY_EXP_EXP = 2 };
+enum { DECAY_PER_HEAD = 0, DECAY_SIGMOID_ROOT = 1, DECAY_EXP_EXP = 2, DECAY_READY = 3 };   // READY: z holds the decays themselves
+typedef __attribute__((ext_vector_type(4))) float scan_f32x4;
 enum { GATE_SILU = 0, GATE_SIGMOID = 1 };
 
 #define SCAN_THREADS 256
@@ -61,18 +62,22 @@ struct ScanArgs {
 
 // One block per (entry, head, slice of PC value channels).  Thread (r, p) keeps the NPT state rows n = r * NPT ..
 // of column p in registers; R = 256 / PC such threads cover R * NPT >= N rows (rows from N on see k = q = 0).  The
-// entry's tokens are walked in chunks of SCAN_CHUNK: the chunk's q, k, decays and v are staged in shared memory
-// (activation, scale and the decay's function applied once on the way), the next chunk's raw values are fetched
-// into registers before the current chunk is worked on and written to the other buffer afterwards.  Every thread
-// leaves one partial sum per token; after one barrier the block adds each token's R partial sums in the order of r.
-template <int PC, int NPT, bool BEFORE>
+// entry's tokens are walked in chunks of CH: the chunk's q, k, decays and v are staged in shared memory
+// (activation, scale and the decay's function applied on the way unless a pass before has applied them), the next
+// chunk's raw values are fetched into registers before the current chunk is worked on and written to the other
+// buffer afterwards.  A token's staged values are read one token ahead of the arithmetic that uses them.  Every
+// thread leaves one partial sum per token; after one barrier the block adds each token's R partial sums in the
+// order of r.  CH = 1 serves steps of single tokens: little shared memory, so that many blocks of a compute unit
+// have their state rows on the way at once.
+template <int PC, int NPT, bool BEFORE, int CH>
 __global__ void __launch_bounds__(SCAN_THREADS)
 decay_scan_kernel(const ScanArgs a) {
   constexpr int R = SCAN_THREADS / PC;
   constexpr int NP = R * NPT;                       // padded key channels
   constexpr int ROW = 3 * NP + PC;                  // staged values of a token: q | k | d | v
-  constexpr int PER_BUF = SCAN_CHUNK * ROW;
-  constexpr int PER_TOK = (3 * NP + PC + 15) / 16;  // values each of a token's 16 staging lanes brings
+  constexpr int PER_BUF = CH * ROW;
+  constexpr int LANES = SCAN_THREADS / CH;          // staging lanes of a token
+  constexpr int PER_TOK = (ROW + LANES - 1) / LANES;
   extern __shared__ __attribute__((aligned(16))) float shared[];
   float* part = shared + 2 * PER_BUF;               // [chunk][R][PC]
   const int b = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * PC;
@@ -89,7 +94,7 @@ decay_scan_kernel(const ScanArgs a) {
     u[i] = (BEFORE && a.bonus != nullptr && n < N) ? a.bonus[(size_t)h * N + n] : 0.f;
   }
   const float head_decay = a.decay_kind == DECAY_PER_HEAD ? a.z[h] : 1.f;
-  const int tl = tid / 16, ln = tid % 16;           // staging: token of the chunk, lane of its 16
+  const int tl = tid / LANES, ln = tid % LANES;     // staging: token of the chunk, lane of its LANES
   float raw[PER_TOK];
   // element e of a token's staged row: [0, NP) q, [NP, 2NP) k, [2NP, 3NP) decay, then PC values of v
   auto fetch = [&](int c0) __attribute__((always_inline)) {
@@ -97,7 +102,7 @@ decay_scan_kernel(const ScanArgs a) {
     const bool live = tok < end;
 #pragma unroll
     for (int i = 0; i < PER_TOK; ++i) {
-      const int e = ln + 16 * i;
+      const int e = ln + LANES * i;
       float val = 0.f;
       if (live && e < ROW) {
         if (e < 3 * NP) {
@@ -119,13 +124,15 @@ decay_scan_kernel(const ScanArgs a) {
     float* dst = buf + tl * ROW;
 #pragma unroll
     for (int i = 0; i < PER_TOK; ++i) {
-      const int e = ln + 16 * i;
+      const int e = ln + LANES * i;
       if (e < ROW) {
         float val = raw[i];
         const int which = e < 3 * NP ? e / NP : 3;
         if (which == 2) {
           // tokens past the entry's end and rows past N: decay 1 on a state that takes nothing
-          val = (!live || e % NP >= N) ? 1.f : (a.decay_kind == DECAY_PER_HEAD ? head_decay : decay_of(val, a.decay_kind, a.inv_tau));
+          if (!live || e % NP >= N) val = 1.f;
+          else if (a.decay_kind == DECAY_PER_HEAD) val = head_decay;
+          else if (a.decay_kind != DECAY_READY) val = decay_of(val, a.decay_kind, a.inv_tau);
         } else {
           if (a.silu_inputs) val = exact_silu(val);
           if (which == 0) val *= a.q_scale;
@@ -134,32 +141,69 @@ decay_scan_kernel(const ScanArgs a) {
       }
     }
   };
+  struct TokenIn {
+    float q[NPT], k[NPT], d[NPT];
+    float v;
+  };
+  auto read_token = [&](const float* buf, int t, TokenIn& in) __attribute__((always_inline)) {
+    const float* src = buf + t * ROW + r * NPT;
+    if constexpr (NPT % 4 == 0) {
+#pragma unroll
+      for (int i = 0; i < NPT; i += 4) {
+        const scan_f32x4 qq = *reinterpret_cast<const scan_f32x4*>(src + i);
+        const scan_f32x4 kk = *reinterpret_cast<const scan_f32x4*>(src + NP + i);
+        const scan_f32x4 dd = *reinterpret_cast<const scan_f32x4*>(src + 2 * NP + i);
+        in.q[i] = qq.x, in.q[i + 1] = qq.y, in.q[i + 2] = qq.z, in.q[i + 3] = qq.w;
+        in.k[i] = kk.x, in.k[i + 1] = kk.y, in.k[i + 2] = kk.z, in.k[i + 3] = kk.w;
+        in.d[i] = dd.x, in.d[i + 1] = dd.y, in.d[i + 2] = dd.z, in.d[i + 3] = dd.w;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NPT; ++i) in.q[i] = src[i], in.k[i] = src[NP + i], in.d[i] = src[2 * NP + i];
+    }
+    in.v = buf[t * ROW + 3 * NP + p];
+  };
+  // one token: every row of this thread decays and takes its share of k v^T; returns the thread's part of the output
+  auto move_rows = [&](const TokenIn& in) __attribute__((always_inline)) {
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) {
+      const float kv = in.k[i] * in.v;
+      if (BEFORE) {
+        acc += (s[i] + u[i] * kv) * in.q[i];
+        s[i] = in.d[i] * s[i] + kv;
+      } else {
+        s[i] = in.d[i] * s[i] + kv;
+        acc += s[i] * in.q[i];
+      }
+    }
+    return acc;
+  };
   fetch(first);
   put(first, shared);
   shared_memory_barrier();
   int turn = 0;
-  for (int c0 = first; c0 < end; c0 += SCAN_CHUNK) {
+  for (int c0 = first; c0 < end; c0 += CH) {
     const float* buf = shared + turn * PER_BUF;
-    const bool more = c0 + SCAN_CHUNK < end;
-    if (more) fetch(c0 + SCAN_CHUNK);
-    const int n_tok = end - c0 < SCAN_CHUNK ? end - c0 : SCAN_CHUNK;
-    for (int t = 0; t < n_tok; ++t) {
-      const float* in = buf + t * ROW + r * NPT;
-      const float vp = buf[t * ROW + 3 * NP + p];
-      float acc = 0.f;
-#pragma unroll
-      for (int i = 0; i < NPT; ++i) {
-        const float qn = in[i], kn = in[NP + i], dn = in[2 * NP + i];
-        const float kv = kn * vp;
-        if (BEFORE) {
-          acc += (s[i] + u[i] * kv) * qn;
-          s[i] = dn * s[i] + kv;
-        } else {
-          s[i] = dn * s[i] + kv;
-          acc += s[i] * qn;
-        }
+    const bool more = c0 + CH < end;
+    if (more) fetch(c0 + CH);
+    const int n_tok = end - c0 < CH ? end - c0 : CH;
+    if constexpr (CH == 1) {
+      TokenIn in;
+      read_token(buf, 0, in);
+      part[r * PC + p] = move_rows(in);
+    } else {
+      // two sets of registers take turns: a token's values are read while the token before is worked on (tokens
+      // past the entry's end were staged with k = 0 and a decay of one: they change nothing)
+      const int t_end = (n_tok + 1) & ~1;
+      TokenIn in_a, in_b;
+      read_token(buf, 0, in_a);
+      for (int t = 0; t < t_end; t += 2) {
+        read_token(buf, t + 1, in_b);
+        part[(t * R + r) * PC + p] = move_rows(in_a);
+        read_token(buf, t + 2 < CH ? t + 2 : CH - 1, in_a);
+        part[((t + 1) * R + r) * PC + p] = move_rows(in_b);
       }
-      part[(t * R + r) * PC + p] = acc;
     }
     shared_memory_barrier();
     for (int e = tid; e < n_tok * PC; e += SCAN_THREADS) {
@@ -171,7 +215,7 @@ decay_scan_kernel(const ScanArgs a) {
         a.out[(size_t)(c0 + t) * a.heads * P + h * P + p0 + pp] = sum;
       }
     }
-    if (more) put(c0 + SCAN_CHUNK, shared + (1 - turn) * PER_BUF);
+    if (more) put(c0 + CH, shared + (1 - turn) * PER_BUF);
     shared_memory_barrier();
     turn = 1 - turn;
   }
@@ -184,45 +228,46 @@ decay_scan_kernel(const ScanArgs a) {
   }
 }
 
-template <int PC, int NPT>
-static int launch_decay_scan(const ScanArgs& a, int B_, hipStream_t stream) {
+template <int PC, int NPT, bool BEFORE, int CH>
+static int launch_decay_scan_as(const ScanArgs& a, int B_, hipStream_t stream) {
   constexpr int R = SCAN_THREADS / PC, NP = R * NPT;
-  constexpr size_t need = (2 * (size_t)SCAN_CHUNK * (3 * NP + PC) + (size_t)SCAN_CHUNK * R * PC) * sizeof(float);
+  constexpr size_t need = (2 * (size_t)CH * (3 * NP + PC) + (size_t)CH * R * PC) * sizeof(float);
   static_assert(need <= 160 * 1024, "a block's staging fits the shared memory of a compute unit");
-  const dim3 grid(B_, a.heads, (a.P + PC - 1) / PC);
-  if (a.before) {
-    if (need > 48 * 1024) {
-      const hipError_t e = hipFuncSetAttribute((const void*)decay_scan_kernel<PC, NPT, true>,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)need);
-      if (e != hipSuccess) return (int)e;
-    }
-    hipLaunchKernelGGL((decay_scan_kernel<PC, NPT, true>), grid, dim3(SCAN_THREADS), need, stream, a);
-  } else {
-    if (need > 48 * 1024) {
-      const hipError_t e = hipFuncSetAttribute((const void*)decay_scan_kernel<PC, NPT, false>,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)need);
-      if (e != hipSuccess) return (int)e;
-    }
-    hipLaunchKernelGGL((decay_scan_kernel<PC, NPT, false>), grid, dim3(SCAN_THREADS), need, stream, a);
+  if (need > 48 * 1024) {
+    const hipError_t e = hipFuncSetAttribute((const void*)decay_scan_kernel<PC, NPT, BEFORE, CH>,
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)need);
+    if (e != hipSuccess) return (int)e;
   }
+  hipLaunchKernelGGL((decay_scan_kernel<PC, NPT, BEFORE, CH>), dim3(B_, a.heads, (a.P + PC - 1) / PC), dim3(SCAN_THREADS),
+                     need, stream, a);
   ULLM_LAUNCH_CHECK();
 }
 
+template <int PC, int NPT>
+static int launch_decay_scan(const ScanArgs& a, int B_, bool single, hipStream_t stream) {
+  if (a.before) return single ? launch_decay_scan_as<PC, NPT, true, 1>(a, B_, stream)
+                              : launch_decay_scan_as<PC, NPT, true, SCAN_CHUNK>(a, B_, stream);
+  return single ? launch_decay_scan_as<PC, NPT, false, 1>(a, B_, stream)
+                : launch_decay_scan_as<PC, NPT, false, SCAN_CHUNK>(a, B_, stream);
+}
+
+// max_len: the most tokens any entry brings (1: a step of single tokens).
 extern "C" int ullm_decay_scan(const float* q, int q_ld, const float* k, int k_ld, const float* v, int v_ld, const float* z,
                                int z_ld, int decay_kind, float tau, const float* bonus, int silu_inputs, float q_scale,
                                int before, float* state, long long state_stride, long long state_off,
                                const int* q_start, const int* entry_slot, float* out, int B_, int heads, int N, int P,
-                               int write_state, hipStream_t stream) {
+                               int write_state, int max_len, hipStream_t stream) {
   if (B_ <= 0) return 0;
   if (heads <= 0 || N <= 0 || P <= 0 || N > 256) return ULLM_ERR_SHAPE;
-  if (decay_kind < DECAY_PER_HEAD || decay_kind > DECAY_EXP_EXP || z == nullptr) return ULLM_ERR_UNSUPPORTED;
+  if (decay_kind < DECAY_PER_HEAD || decay_kind > DECAY_READY || z == nullptr) return ULLM_ERR_UNSUPPORTED;
   if (decay_kind == DECAY_SIGMOID_ROOT && !(tau > 0.f)) return ULLM_ERR_UNSUPPORTED;
   ScanArgs a;
   a.q = q, a.k = k, a.v = v, a.z = z, a.bonus = bonus, a.state = state, a.state_stride = state_stride, a.state_off = state_off;
   a.q_start = q_start, a.entry_slot = entry_slot, a.out = out, a.q_ld = q_ld, a.k_ld = k_ld, a.v_ld = v_ld, a.z_ld = z_ld;
   a.heads = heads, a.N = N, a.P = P, a.decay_kind = decay_kind, a.silu_inputs = silu_inputs, a.before = before;
   a.write_state = write_state, a.q_scale = q_scale, a.inv_tau = decay_kind == DECAY_SIGMOID_ROOT ? 1.f / tau : 1.f;
-#define SCAN_GO(PC, NPT) return launch_decay_scan<PC, NPT>(a, B_, stream)
+  const bool single = max_len == 1;
+#define SCAN_GO(PC, NPT) return launch_decay_scan<PC, NPT>(a, B_, single, stream)
   // whole rows of 64 value channels a block where there are blocks enough without slicing the heads (a step of
   // many requests: the state's rows then move as whole lines); else slices of 16
   if (P % 64 == 0 && N <= 128 && (long long)B_ * heads >= 1024) {
@@ -238,13 +283,47 @@ extern "C" int ullm_decay_scan(const float* q, int q_ld, const float* k, int k_l
 #undef SCAN_GO
 }
 
+// ------------------------------------------------------------------ the inputs' functions, ahead of the recurrence
+// For steps of many tokens: silu over a column range of the projection's rows and the decay's function over the raw
+// decays, both in place, once per value (the recurrence's blocks, one per slice of value channels, would each apply
+// them again).  The same functions as inside the recurrence: a value has the same bits whichever applied them.
+__global__ void __launch_bounds__(256)
+decay_prepare_kernel(float* __restrict__ x, int x_ld, int x_cols, float* __restrict__ z, int z_ld, int z_cols, int decay_kind,
+                     float inv_tau, int T_) {
+  const int cols = x_cols + z_cols;
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)T_ * cols) return;
+  const int t = (int)(i / cols), c = (int)(i % cols);
+  if (c < x_cols) {
+    float* p = x + (size_t)t * x_ld + c;
+    *p = exact_silu(*p);
+  } else {
+    float* p = z + (size_t)t * z_ld + (c - x_cols);
+    *p = decay_of(*p, decay_kind, inv_tau);
+  }
+}
+
+extern "C" int ullm_decay_prepare(float* x, int x_ld, int x_cols, float* z, int z_ld, int z_cols, int decay_kind, float tau,
+                                  int T_, hipStream_t stream) {
+  if (T_ <= 0 || x_cols + z_cols <= 0) return 0;
+  if (x_cols < 0 || z_cols < 0 || (x_cols && !x) || (z_cols && !z)) return ULLM_ERR_SHAPE;
+  if (z_cols && decay_kind != DECAY_SIGMOID_ROOT && decay_kind != DECAY_EXP_EXP) return ULLM_ERR_UNSUPPORTED;
+  if (z_cols && decay_kind == DECAY_SIGMOID_ROOT && !(tau > 0.f)) return ULLM_ERR_UNSUPPORTED;
+  const size_t n = (size_t)T_ * (x_cols + z_cols);
+  hipLaunchKernelGGL(decay_prepare_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, x_ld, x_cols, z, z_ld,
+                     z_cols, decay_kind, decay_kind == DECAY_SIGMOID_ROOT ? 1.f / tau : 1.f, T_);
+  ULLM_LAUNCH_CHECK();
+}
+
 // ------------------------------------------------------------------ token shift
 // out[m, t, :] = x[t] + (prev(t) - x[t]) * mu[m] for m < M, with prev(t) the row before t in its entry or, for an
 // entry's first token, what the state row holds (the last row of the step before; zeros at a request's start).
 // The block of an entry's first token then puts the entry's last row into the state row: a thread reads the old
 // value of a column before it writes the new one.
-template <typename T>
-__global__ void __launch_bounds__(256)
+// V columns a thread (4 where the rows allow 16-byte pieces, 8-byte ones of bfloat16), as many threads as the row
+// has such pieces, up to 1024.
+template <typename T, int V>
+__global__ void __launch_bounds__(1024)
 token_shift_kernel(const T* __restrict__ x, const float* __restrict__ mu, float* __restrict__ state,
                    long long state_stride, long long state_off, const int* __restrict__ token_entry,
                    const int* __restrict__ q_start, const int* __restrict__ entry_slot, T* __restrict__ out, int T_,
@@ -255,12 +334,23 @@ token_shift_kernel(const T* __restrict__ x, const float* __restrict__ mu, float*
   const bool head = t == first;
   float* row = state + (size_t)entry_slot[b] * state_stride + state_off;
   const int last = q_start[b + 1] - 1;
-  for (int col = threadIdx.x; col < H; col += 256) {
-    const float cur = ld_f32(x + (size_t)t * H + col);
-    const float prev = head ? row[col] : ld_f32(x + (size_t)(t - 1) * H + col);
-    const float diff = prev - cur;
-    for (int m = 0; m < M; ++m) st_f32(out + ((size_t)m * T_ + t) * H + col, cur + diff * mu[(size_t)m * H + col]);
-    if (head && write_state) row[col] = ld_f32(x + (size_t)last * H + col);
+  for (int col = V * threadIdx.x; col < H; col += V * blockDim.x) {
+    float cur[V], diff[V], keep[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      cur[j] = ld_f32(x + (size_t)t * H + col + j);
+      const float prev = head ? row[col + j] : ld_f32(x + (size_t)(t - 1) * H + col + j);
+      diff[j] = prev - cur[j];
+      keep[j] = (head && write_state) ? ld_f32(x + (size_t)last * H + col + j) : 0.f;
+    }
+    for (int m = 0; m < M; ++m) {
+#pragma unroll
+      for (int j = 0; j < V; ++j) st_f32(out + ((size_t)m * T_ + t) * H + col + j, cur[j] + diff[j] * mu[(size_t)m * H + col + j]);
+    }
+    if (head && write_state) {
+#pragma unroll
+      for (int j = 0; j < V; ++j) row[col + j] = keep[j];
+    }
   }
 }
 
@@ -269,37 +359,72 @@ extern "C" int ullm_token_shift(const void* x, const float* mu, float* state, lo
                                 int H, int M, int write_state, int dtype, hipStream_t stream) {
   if (T_ <= 0) return 0;
   if (H < 1 || M < 1) return ULLM_ERR_SHAPE;
-  if (dtype == ULLM_F32)
-    hipLaunchKernelGGL(token_shift_kernel<float>, dim3(T_), dim3(256), 0, stream, (const float*)x, mu, state, state_stride,
-                       state_off, token_entry, q_start, entry_slot, (float*)out, T_, H, M, write_state);
-  else if (dtype == ULLM_BF16)
-    hipLaunchKernelGGL(token_shift_kernel<bf16_t>, dim3(T_), dim3(256), 0, stream, (const bf16_t*)x, mu, state, state_stride,
-                       state_off, token_entry, q_start, entry_slot, (bf16_t*)out, T_, H, M, write_state);
+  const bool vec = H % 4 == 0;
+  const int pieces = vec ? H / 4 : H;
+  int threads = 64;
+  while (threads < pieces && threads < 1024) threads *= 2;
+#define SHIFT_GO(TT, V) hipLaunchKernelGGL((token_shift_kernel<TT, V>), dim3(T_), dim3(threads), 0, stream, (const TT*)x, mu, state, \
+    state_stride, state_off, token_entry, q_start, entry_slot, (TT*)out, T_, H, M, write_state)
+  if (dtype == ULLM_F32) { if (vec) SHIFT_GO(float, 4); else SHIFT_GO(float, 1); }
+  else if (dtype == ULLM_BF16) { if (vec) SHIFT_GO(bf16_t, 4); else SHIFT_GO(bf16_t, 1); }
   else return ULLM_ERR_DTYPE;
+#undef SHIFT_GO
   ULLM_LAUNCH_CHECK();
 }
 
 // ------------------------------------------------------------------ norm of the outputs, gain and gate
 // The row o [width] is cut into `parts` equal parts (the heads, or one part); each is divided by its root mean
 // square (eps inside the root), multiplied by gain[c % gain_len] (a gain per value channel shared by the heads, or
-// one per column) and by silu or sigmoid of the gate's raw value g[t, c].  A wave per part, parts taken in turn.
+// one per column) and by silu or sigmoid of the gate's raw value g[t, c].  Parts of up to 1024 values: a wave per
+// (token, part), every lane's values in registers between the sum of squares and the scaling; longer parts: a block.
+#define NORM_PER_LANE 16
 template <typename TO>
 __global__ void __launch_bounds__(256)
-gated_unit_norm_kernel(const float* __restrict__ o, const float* __restrict__ g, int g_ld, const float* __restrict__ gain,
-                       int gain_len, float eps, int gate_kind, TO* __restrict__ out, int width, int parts) {
-  const int t = blockIdx.x, lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+gated_unit_norm_wave_kernel(const float* __restrict__ o, const float* __restrict__ g, int g_ld, const float* __restrict__ gain,
+                            int gain_len, float eps, int gate_kind, TO* __restrict__ out, int T_, int width, int parts) {
+  const int lane = threadIdx.x % WAVE;
+  const long long item = (long long)blockIdx.x * (256 / WAVE) + threadIdx.x / WAVE;
+  if (item >= (long long)T_ * parts) return;
+  const int t = (int)(item / parts), part = (int)(item % parts);
   const int size = width / parts;
-  for (int part = wave; part < parts; part += 256 / WAVE) {
-    const float* src = o + (size_t)t * width + (size_t)part * size;
-    float sq = 0.f;
-    for (int c = lane; c < size; c += WAVE) sq += src[c] * src[c];
-    const float r = 1.f / sqrtf(wave_sum(sq) / (float)size + eps);
-    for (int c = lane; c < size; c += WAVE) {
+  const float* src = o + (size_t)t * width + (size_t)part * size;
+  float v[NORM_PER_LANE], z[NORM_PER_LANE];
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < NORM_PER_LANE; ++i) {
+    const int c = lane + WAVE * i;
+    v[i] = c < size ? src[c] : 0.f;
+    z[i] = c < size ? g[(size_t)t * g_ld + part * size + c] : 0.f;
+    sq += v[i] * v[i];
+  }
+  const float r = 1.f / sqrtf(wave_sum(sq) / (float)size + eps);
+#pragma unroll
+  for (int i = 0; i < NORM_PER_LANE; ++i) {
+    const int c = lane + WAVE * i;
+    if (c < size) {
       const int col = part * size + c;
-      const float z = g[(size_t)t * g_ld + col];
-      const float gate = gate_kind == GATE_SIGMOID ? 1.f / (1.f + expf(-z)) : exact_silu(z);
-      st_f32(out + (size_t)t * width + col, src[c] * r * gain[col % gain_len] * gate);
+      const float gate = gate_kind == GATE_SIGMOID ? 1.f / (1.f + expf(-z[i])) : exact_silu(z[i]);
+      st_f32(out + (size_t)t * width + col, v[i] * r * gain[col % gain_len] * gate);
     }
+  }
+}
+
+template <typename TO>
+__global__ void __launch_bounds__(1024)
+gated_unit_norm_block_kernel(const float* __restrict__ o, const float* __restrict__ g, int g_ld, const float* __restrict__ gain,
+                             int gain_len, float eps, int gate_kind, TO* __restrict__ out, int width, int parts) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x / parts, part = blockIdx.x % parts;
+  const int size = width / parts;
+  const float* src = o + (size_t)t * width + (size_t)part * size;
+  float sq = 0.f;
+  for (int c = threadIdx.x; c < size; c += blockDim.x) sq += src[c] * src[c];
+  const float r = 1.f / sqrtf(block_sum(sq, scratch) / (float)size + eps);
+  for (int c = threadIdx.x; c < size; c += blockDim.x) {
+    const int col = part * size + c;
+    const float z = g[(size_t)t * g_ld + col];
+    const float gate = gate_kind == GATE_SIGMOID ? 1.f / (1.f + expf(-z)) : exact_silu(z);
+    st_f32(out + (size_t)t * width + col, src[c] * r * gain[col % gain_len] * gate);
   }
 }
 
@@ -309,12 +434,27 @@ extern "C" int ullm_gated_unit_norm(const float* o, const float* g, int g_ld, co
   if (T_ <= 0) return 0;
   if (width < 1 || parts < 1 || width % parts || gain_len < 1 || width % gain_len) return ULLM_ERR_SHAPE;
   if (gate_kind != GATE_SILU && gate_kind != GATE_SIGMOID) return ULLM_ERR_UNSUPPORTED;
-  if (out_dtype == ULLM_F32)
-    hipLaunchKernelGGL(gated_unit_norm_kernel<float>, dim3(T_), dim3(256), 0, stream, o, g, g_ld, gain, gain_len, eps,
-                       gate_kind, (float*)out, width, parts);
-  else if (out_dtype == ULLM_BF16)
-    hipLaunchKernelGGL(gated_unit_norm_kernel<bf16_t>, dim3(T_), dim3(256), 0, stream, o, g, g_ld, gain, gain_len, eps,
-                       gate_kind, (bf16_t*)out, width, parts);
-  else return ULLM_ERR_DTYPE;
+  if (out_dtype != ULLM_F32 && out_dtype != ULLM_BF16) return ULLM_ERR_DTYPE;
+  const int size = width / parts;
+  if (size <= WAVE * NORM_PER_LANE) {
+    const long long items = (long long)T_ * parts;
+    const dim3 grid((unsigned)((items + 3) / 4));
+    if (out_dtype == ULLM_F32)
+      hipLaunchKernelGGL(gated_unit_norm_wave_kernel<float>, grid, dim3(256), 0, stream, o, g, g_ld, gain, gain_len, eps,
+                         gate_kind, (float*)out, T_, width, parts);
+    else
+      hipLaunchKernelGGL(gated_unit_norm_wave_kernel<bf16_t>, grid, dim3(256), 0, stream, o, g, g_ld, gain, gain_len, eps,
+                         gate_kind, (bf16_t*)out, T_, width, parts);
+  } else {
+    int threads = 256;
+    while (threads < size / 4 && threads < 1024) threads *= 2;
+    const dim3 grid((unsigned)((long long)T_ * parts));
+    if (out_dtype == ULLM_F32)
+      hipLaunchKernelGGL(gated_unit_norm_block_kernel<float>, grid, dim3(threads), 0, stream, o, g, g_ld, gain, gain_len, eps,
+                         gate_kind, (float*)out, width, parts);
+    else
+      hipLaunchKernelGGL(gated_unit_norm_block_kernel<bf16_t>, grid, dim3(threads), 0, stream, o, g, g_ld, gain, gain_len, eps,
+                         gate_kind, (bf16_t*)out, width, parts);
+  }
   ULLM_LAUNCH_CHECK();
 }

@@ -9,7 +9,6 @@
 #include "common.h"
 
 #define STREAMS_MAX 8
-#define STREAMS_THREADS 256
 enum { NORM_RMS = 0, NORM_LAYER = 1 };
 
 struct StreamCoeffs {
@@ -18,77 +17,138 @@ struct StreamCoeffs {
   float mix[STREAMS_MAX * STREAMS_MAX];
 };
 
-template <typename TY, typename TO>
-__global__ void __launch_bounds__(STREAMS_THREADS)
+// V values a thread and turn: 4 where rows and pointers allow 16-byte accesses (8-byte ones of bfloat16), else 1.
+template <typename T, int V>
+struct RowPiece {
+  float v[V];
+};
+template <int V>
+__device__ __forceinline__ RowPiece<float, V> load_piece(const float* p) {
+  RowPiece<float, V> r;
+  if constexpr (V == 4) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    r.v[0] = t.x, r.v[1] = t.y, r.v[2] = t.z, r.v[3] = t.w;
+  } else {
+    r.v[0] = *p;
+  }
+  return r;
+}
+template <int V>
+__device__ __forceinline__ RowPiece<float, V> load_piece(const bf16_t* p) {
+  RowPiece<float, V> r;
+  if constexpr (V == 4) {
+    const uint2 t = *reinterpret_cast<const uint2*>(p);
+    r.v[0] = __uint_as_float(t.x << 16), r.v[1] = __uint_as_float(t.x & 0xffff0000u);
+    r.v[2] = __uint_as_float(t.y << 16), r.v[3] = __uint_as_float(t.y & 0xffff0000u);
+  } else {
+    r.v[0] = bf16_bits_to_f32(*p);
+  }
+  return r;
+}
+template <int V>
+__device__ __forceinline__ void store_piece(float* p, const float* v) {
+  if constexpr (V == 4) *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  else *p = v[0];
+}
+template <int V>
+__device__ __forceinline__ void store_piece(bf16_t* p, const float* v) {
+  if constexpr (V == 4) *reinterpret_cast<uint2*>(p) = make_uint2(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]));
+  else *p = f32_to_bf16_bits(v[0]);
+}
+
+// One block per token, as many threads as the row has pieces (up to 1024): with rows of up to 4096 values every
+// thread has all its loads on the way at once.
+template <typename TY, typename TO, int V>
+__global__ void __launch_bounds__(1024)
 streams_step_kernel(float* __restrict__ streams, const TY* __restrict__ ya, const TY* __restrict__ yb, float a, float b,
                     const float* __restrict__ mix, const float* __restrict__ out_w, float mult,
                     const float* __restrict__ in_w, const float* __restrict__ gain, float eps, int kind,
                     TO* __restrict__ normed, const int* __restrict__ rows, int T, int H, int S, int write_back) {
-  extern __shared__ float u_row[];                  // [H]: the mix the next sublayer reads
+  extern __shared__ __attribute__((aligned(16))) float u_row[];      // [H]: the mix the next sublayer reads
   __shared__ float scratch[16];
   __shared__ StreamCoeffs c;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, nthreads = blockDim.x;
   const int t = rows ? rows[blockIdx.x] : blockIdx.x;
   if (tid < S) {
     c.in[tid] = in_w ? in_w[tid] : 0.f;
     c.out[tid] = out_w ? out_w[tid] : 0.f;
   }
   if (mix != nullptr)
-    for (int e = tid; e < S * S; e += STREAMS_THREADS) c.mix[e] = mix[e];
+    for (int e = tid; e < S * S; e += nthreads) c.mix[e] = mix[e];
   __syncthreads();
   const bool has_branch = ya != nullptr;
   float sum = 0.f;
-  for (int col = tid; col < H; col += STREAMS_THREADS) {
-    float x[STREAMS_MAX];
+  for (int col = V * tid; col < H; col += V * nthreads) {
+    RowPiece<float, V> x[STREAMS_MAX];
 #pragma unroll
     for (int s = 0; s < STREAMS_MAX; ++s)
-      if (s < S) x[s] = streams[((size_t)s * T + t) * H + col];
+      if (s < S) x[s] = load_piece<V>(streams + ((size_t)s * T + t) * H + col);
     if (has_branch) {
-      float y = a * ld_f32(ya + (size_t)t * H + col);
-      if (yb != nullptr) y += b * ld_f32(yb + (size_t)t * H + col);
-      y *= mult;
-      float nx[STREAMS_MAX];
+      RowPiece<float, V> y = load_piece<V>(ya + (size_t)t * H + col);
+      if (yb != nullptr) {
+        const RowPiece<float, V> y2 = load_piece<V>(yb + (size_t)t * H + col);
+#pragma unroll
+        for (int j = 0; j < V; ++j) y.v[j] = a * y.v[j] + b * y2.v[j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j) y.v[j] = a * y.v[j];
+      }
+      RowPiece<float, V> nx[STREAMS_MAX];
 #pragma unroll
       for (int to = 0; to < STREAMS_MAX; ++to) {
         if (to < S) {
-          float v = 0.f;
 #pragma unroll
-          for (int s = 0; s < STREAMS_MAX; ++s)
-            if (s < S) v += c.mix[s * S + to] * x[s];
-          nx[to] = v + c.out[to] * y;
+          for (int j = 0; j < V; ++j) {
+            float v = 0.f;
+#pragma unroll
+            for (int s = 0; s < STREAMS_MAX; ++s)
+              if (s < S) v += c.mix[s * S + to] * x[s].v[j];
+            nx[to].v[j] = v + c.out[to] * (mult * y.v[j]);
+          }
         }
       }
 #pragma unroll
       for (int s = 0; s < STREAMS_MAX; ++s) {
         if (s < S) {
           x[s] = nx[s];
-          if (write_back) streams[((size_t)s * T + t) * H + col] = nx[s];
+          if (write_back) store_piece<V>(streams + ((size_t)s * T + t) * H + col, nx[s].v);
         }
       }
     }
     if (gain != nullptr) {
-      float u = 0.f;
 #pragma unroll
-      for (int s = 0; s < STREAMS_MAX; ++s)
-        if (s < S) u += c.in[s] * x[s];
-      u_row[col] = u;
-      sum += kind == NORM_LAYER ? u : u * u;
+      for (int j = 0; j < V; ++j) {
+        float u = 0.f;
+#pragma unroll
+        for (int s = 0; s < STREAMS_MAX; ++s)
+          if (s < S) u += c.in[s] * x[s].v[j];
+        u_row[col + j] = u;
+        sum += kind == NORM_LAYER ? u : u * u;
+      }
     }
   }
   if (gain == nullptr) return;
   TO* dst = normed + (size_t)blockIdx.x * H;
+  float mean = 0.f, r;
   if (kind == NORM_LAYER) {
-    const float mean = block_sum(sum, scratch) / (float)H;
+    mean = block_sum(sum, scratch) / (float)H;
     float dev = 0.f;
-    for (int col = tid; col < H; col += STREAMS_THREADS) {
-      const float d = u_row[col] - mean;
-      dev += d * d;
+    for (int col = V * tid; col < H; col += V * nthreads) {
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        const float d = u_row[col + j] - mean;
+        dev += d * d;
+      }
     }
-    const float r = 1.f / sqrtf(block_sum(dev, scratch) / (float)H + eps);
-    for (int col = tid; col < H; col += STREAMS_THREADS) st_f32(dst + col, (u_row[col] - mean) * r * gain[col]);
+    r = 1.f / sqrtf(block_sum(dev, scratch) / (float)H + eps);
   } else {
-    const float r = 1.f / sqrtf(block_sum(sum, scratch) / (float)H + eps);
-    for (int col = tid; col < H; col += STREAMS_THREADS) st_f32(dst + col, u_row[col] * r * gain[col]);
+    r = 1.f / sqrtf(block_sum(sum, scratch) / (float)H + eps);
+  }
+  for (int col = V * tid; col < H; col += V * nthreads) {
+    float o[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) o[j] = (u_row[col + j] - mean) * r * gain[col + j];
+    store_piece<V>(dst + col, o);
   }
 }
 
@@ -107,23 +167,30 @@ extern "C" int ullm_streams_step(float* streams, const void* ya, const void* yb,
   const size_t shared = gain ? (size_t)H * sizeof(float) : 0;
   if (shared > 160 * 1024 - 4096) return ULLM_ERR_SHAPE;
   const int write_back = rows == nullptr ? 1 : 0;
-#define STREAMS_GO(TY, TO)                                                                                           \
+  const bool vec = H % 4 == 0 && ((uintptr_t)streams % 16) == 0 && ((uintptr_t)ya % 16) == 0 && ((uintptr_t)yb % 16) == 0 &&
+                   ((uintptr_t)normed % 16) == 0;
+  const int pieces = vec ? H / 4 : H;
+  int threads = 64;
+  while (threads < pieces && threads < 1024) threads *= 2;
+#define STREAMS_GO_V(TY, TO, V)                                                                                      \
   do {                                                                                                               \
     if (shared > 48 * 1024) {                                                                                        \
-      const hipError_t e = hipFuncSetAttribute((const void*)streams_step_kernel<TY, TO>,                             \
+      const hipError_t e = hipFuncSetAttribute((const void*)streams_step_kernel<TY, TO, V>,                          \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shared);             \
       if (e != hipSuccess) return (int)e;                                                                            \
     }                                                                                                                \
-    hipLaunchKernelGGL((streams_step_kernel<TY, TO>), dim3(n), dim3(STREAMS_THREADS), shared, stream, streams,       \
+    hipLaunchKernelGGL((streams_step_kernel<TY, TO, V>), dim3(n), dim3(threads), shared, stream, streams,            \
                        (const TY*)ya, (const TY*)yb, a, b, mix, out_w, mult, in_w, gain, eps, kind, (TO*)normed,     \
                        rows, T_, H, S, write_back);                                                                  \
   } while (0)
+#define STREAMS_GO(TY, TO) do { if (vec) STREAMS_GO_V(TY, TO, 4); else STREAMS_GO_V(TY, TO, 1); } while (0)
   if (y_dtype == ULLM_F32 && out_dtype == ULLM_F32) STREAMS_GO(float, float);
   else if (y_dtype == ULLM_F32 && out_dtype == ULLM_BF16) STREAMS_GO(float, bf16_t);
   else if (y_dtype == ULLM_BF16 && out_dtype == ULLM_F32) STREAMS_GO(bf16_t, float);
   else if (y_dtype == ULLM_BF16 && out_dtype == ULLM_BF16) STREAMS_GO(bf16_t, bf16_t);
   else return ULLM_ERR_DTYPE;
 #undef STREAMS_GO
+#undef STREAMS_GO_V
   ULLM_LAUNCH_CHECK();
 }
 

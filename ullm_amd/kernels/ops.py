@@ -595,7 +595,7 @@ def weighted_sum(x: torch.Tensor, y: torch.Tensor, a: float, b: float) -> torch.
 
 # ---------------------------------------------------------------------------------- recurrences with decays
 
-DECAY_PER_HEAD, DECAY_SIGMOID_ROOT, DECAY_EXP_EXP = 0, 1, 2      # how a recurrence's decays come about
+DECAY_PER_HEAD, DECAY_SIGMOID_ROOT, DECAY_EXP_EXP, DECAY_READY = 0, 1, 2, 3      # how a recurrence's decays come about
 GATE_SILU, GATE_SIGMOID = 0, 1
 DECAY_SCAN_MAX_KEYS = 256
 
@@ -608,14 +608,16 @@ def _f32_rows(t: torch.Tensor, name: str, T: int, cols: int) -> None:
 def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, decay_kind: int,
                state: torch.Tensor, state_off: int, q_start: torch.Tensor, entry_slot: torch.Tensor, n_entries: int,
                heads: int, key_dim: int, value_dim: int, tau: float = 1.0, bonus: Optional[torch.Tensor] = None,
-               silu_inputs: bool = False, q_scale: float = 1.0, write_state: bool = True) -> torch.Tensor:
+               silu_inputs: bool = False, q_scale: float = 1.0, write_state: bool = True, max_len: int = 0) -> torch.Tensor:
     """A recurrence per head over each entry's tokens, with the head's state S [key_dim, value_dim] (float32, at
     ``state[slot, state_off + head * key_dim * value_dim ..]``): S = diag(d) S + k v^T and o = S^T q after the
     update, or with ``bonus`` (float32 [heads, key_dim]) o = (S + diag(bonus) k v^T)^T q before it.  ``q``, ``k``
     (float32 [T, heads * key_dim]) and ``v`` (float32 [T, heads * value_dim]) may be column ranges of wider rows; with
     ``silu_inputs`` they go through silu first; q is multiplied by ``q_scale``.  The decays d: ``decay`` float32
     [heads] (DECAY_PER_HEAD: one constant a head) or raw values z float32 [T, heads * key_dim] with d =
-    sigmoid(z)^(1/tau) (DECAY_SIGMOID_ROOT) or exp(-exp(z)) (DECAY_EXP_EXP).  Returns o float32 [T, heads * value_dim]."""
+    sigmoid(z)^(1/tau) (DECAY_SIGMOID_ROOT) or exp(-exp(z)) (DECAY_EXP_EXP), or the decays themselves (DECAY_READY:
+    :func:`decay_prepare` has been over them).  ``max_len``: the most tokens any entry brings, if known (1: a step of
+    single tokens takes a variant of the kernel made for it).  Returns o float32 [T, heads * value_dim]."""
     T = q.shape[0]
     _f32_rows(q, "q", T, heads * key_dim)
     _f32_rows(k, "k", T, heads * key_dim)
@@ -625,7 +627,7 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.T
         _need(decay.dtype == torch.float32 and decay.numel() == heads and decay.is_contiguous(), "decay must be float32 [heads]")
         z_ld = 0
     else:
-        _need(decay_kind in (DECAY_SIGMOID_ROOT, DECAY_EXP_EXP), "unknown kind of decay")
+        _need(decay_kind in (DECAY_SIGMOID_ROOT, DECAY_EXP_EXP, DECAY_READY), "unknown kind of decay")
         _f32_rows(decay, "decay", T, heads * key_dim)
         z_ld = decay.stride(0)
     if bonus is not None:
@@ -641,8 +643,26 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.T
         _c_int(decay_kind), _c_float(tau), _p(bonus), _c_int(1 if silu_inputs else 0), _c_float(q_scale),
         _c_int(1 if bonus is not None else 0), _p(state), ll(state.stride(0)), ll(state_off), _p(q_start), _p(entry_slot),
         _p(out), _c_int(n_entries), _c_int(heads), _c_int(key_dim), _c_int(value_dim), _c_int(1 if write_state else 0),
-        _stream()), "decay_scan")
+        _c_int(max_len), _stream()), "decay_scan")
     return out
+
+
+DECAY_PREPARE_FROM = 16      # from this many tokens a step on, a pass of its own applies the inputs' functions
+
+
+def decay_prepare(x: Optional[torch.Tensor], decay: Optional[torch.Tensor] = None, decay_kind: int = DECAY_EXP_EXP,
+                  tau: float = 1.0) -> None:
+    """In place, ahead of :func:`decay_scan` in a step of many tokens: silu over ``x`` (float32 [T, columns], may be a
+    column range of wider rows) and the decay's function (``decay_kind``) over the raw decays ``decay`` (float32
+    [T, columns]); either may be None.  The recurrence is then called without ``silu_inputs`` and with DECAY_READY."""
+    T = (x if x is not None else decay).shape[0]
+    for t, nm in ((x, "x"), (decay, "decay")):
+        if t is not None:
+            _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape[0] == T and t.stride(1) == 1, f"{nm} must be float32 [T, columns]")
+    _check(build.load("decay_scan").ullm_decay_prepare(
+        _p(x), _c_int(x.stride(0) if x is not None else 0), _c_int(x.shape[1] if x is not None else 0), _p(decay),
+        _c_int(decay.stride(0) if decay is not None else 0), _c_int(decay.shape[1] if decay is not None else 0),
+        _c_int(decay_kind), _c_float(tau), _c_int(T), _stream()), "decay_prepare")
 
 
 def token_shift(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, state_off: int, token_entry: torch.Tensor,

@@ -92,9 +92,15 @@ class GatedLinearAttention(_DecayMixer):
         proj = linear(x, self.w_in, out_dtype=torch.float32)                        # q | k | v | g
         z = linear(linear(x, self.w_a1, out_dtype=torch.float32), self.w_a2, self.b_a2, out_dtype=torch.float32)
         qk, inner = self.qk, self.inner
-        o = ops.decay_scan(proj[:, :qk], proj[:, qk:2 * qk], proj[:, 2 * qk:2 * qk + inner], z, ops.DECAY_SIGMOID_ROOT,
+        kind = ops.DECAY_SIGMOID_ROOT
+        if x.shape[0] >= ops.DECAY_PREPARE_FROM:
+            # many tokens: the decays' function is applied once per value ahead of the recurrence, not by each of its blocks
+            ops.decay_prepare(None, z, kind, self.tau)
+            kind = ops.DECAY_READY
+        o = ops.decay_scan(proj[:, :qk], proj[:, qk:2 * qk], proj[:, 2 * qk:2 * qk + inner], z, kind,
                            self._rows(cache), 0, ctx.q_start, ctx.entry_slot, ctx.num_entries, self.heads, self.key_dim,
-                           self.value_dim, tau=self.tau, q_scale=self.key_dim ** -0.5, write_state=cache.owner)
+                           self.value_dim, tau=self.tau, q_scale=self.key_dim ** -0.5, write_state=cache.owner,
+                           max_len=ctx.max_q_len)
         y = ops.gated_unit_norm(o, proj[:, 2 * qk + inner:], self.gain, self.norm_eps, self.heads, ops.GATE_SILU, ctx.dtype)
         return linear_into_stream(y, self.w_o, ctx)
 
@@ -129,9 +135,12 @@ class LightningAttention(_DecayMixer):
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
         proj = linear(x, self.w_in, out_dtype=torch.float32)                        # q | k | v | g
         qk, inner = self.qk, self.inner
+        ahead = x.shape[0] >= ops.DECAY_PREPARE_FROM
+        if ahead:
+            ops.decay_prepare(proj[:, :2 * qk + inner])              # silu of q | k | v once per value
         o = ops.decay_scan(proj[:, :qk], proj[:, qk:2 * qk], proj[:, 2 * qk:2 * qk + inner], self.decay, ops.DECAY_PER_HEAD,
                            self._rows(cache), 0, ctx.q_start, ctx.entry_slot, ctx.num_entries, self.heads, self.key_dim,
-                           self.value_dim, silu_inputs=True, write_state=cache.owner)
+                           self.value_dim, silu_inputs=not ahead, write_state=cache.owner, max_len=ctx.max_q_len)
         y = ops.gated_unit_norm(o, proj[:, 2 * qk + inner:], self.gain, self.norm_eps, 1, ops.GATE_SIGMOID, ctx.dtype)
         return linear_into_stream(y, self.w_o, ctx)
 
@@ -178,8 +187,13 @@ class TimeMix(_DecayMixer):
         r, k, v = (linear(blends[i], w, out_dtype=f32) for i, w in enumerate((self.w_r, self.w_k, self.w_v)))
         g = linear(blends[3], self.w_g, out_dtype=f32)
         z = linear(linear(blends[4], self.w_w1, out_dtype=f32, act=ops.ACT_TANH), self.w_w2, self.w0, out_dtype=f32)
-        o = ops.decay_scan(r, k, v, z, ops.DECAY_EXP_EXP, rows, self.carry, ctx.q_start, ctx.entry_slot, ctx.num_entries,
-                           self.heads, self.key_dim, self.value_dim, bonus=self.bonus, write_state=cache.owner)
+        kind = ops.DECAY_EXP_EXP
+        if x.shape[0] >= ops.DECAY_PREPARE_FROM:
+            ops.decay_prepare(None, z, kind)
+            kind = ops.DECAY_READY
+        o = ops.decay_scan(r, k, v, z, kind, rows, self.carry, ctx.q_start, ctx.entry_slot, ctx.num_entries,
+                           self.heads, self.key_dim, self.value_dim, bonus=self.bonus, write_state=cache.owner,
+                           max_len=ctx.max_q_len)
         y = ops.gated_unit_norm(o, g, self.gain, self.norm_eps, self.heads, ops.GATE_SILU, ctx.dtype)
         return linear_into_stream(y, self.w_o, ctx)
 

@@ -259,8 +259,10 @@ def test_portions_of_changing_size(replayers, models, name, dtype, cuts):
     got = run(replayers(name, dtype), "r", toks, cuts)
     agree(models, name, toks, got, dtype)
     if dtype == "float32":
-        # the same operations in the same order on every state element and every sum: the cutting changes no bit
-        assert np.array_equal(got, run(replayers(name, dtype), "r", toks, [75]))
+        # a state element goes through the same operations in the same order however the prompt is cut; a token's output
+        # adds its partial sums in an order that goes by the step's shape (slices of 8, 16 or 64 value channels)
+        whole = run(replayers(name, dtype), "r", toks, [75])
+        assert np.abs(got - whole).max() <= 2e-6 * np.abs(whole).max()
 
 
 @pytest.mark.parametrize("name,dtype", CASES)

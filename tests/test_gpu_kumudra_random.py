@@ -148,7 +148,9 @@ def test_drawn_configurations(seed, tmp_path):
     n0 = sharp["r0"]
     assert worst_error(whole[:n0], want["r0"][:n0]) <= bound["r0"], ("whole", worst_error(whole[:n0], want["r0"][:n0]), bound["r0"])
     assert worst_error(cut[:n0], want["r0"][:n0]) <= bound["r0"], ("cut", worst_error(cut[:n0], want["r0"][:n0]), bound["r0"])
-    assert np.array_equal(whole, cut), "whole and cut differ in 32-bit"      # every sum and every state element is ordered by the token alone
+    # a state element sees the same operations however the prompt is cut; a token's partial sums are added in an order
+    # that goes by the step's shape
+    assert worst_error(cut[:n0], whole[:n0]) <= 3e-6, ("whole and cut differ in 32-bit", worst_error(cut[:n0], whole[:n0]))
     for k in reqs:
         assert worst_error(mixed[k][:sharp[k]], want[k][:sharp[k]]) <= bound[k], (k, worst_error(mixed[k][:sharp[k]], want[k][:sharp[k]]), bound[k])
     # bfloat16: the same schedules.  What rounding does depends on the drawn model (up to twenty layer runs: a rounded

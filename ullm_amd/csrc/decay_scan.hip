@@ -65,11 +65,11 @@ struct ScanArgs {
 // entry's tokens are walked in chunks of CH: the chunk's q, k, decays and v are staged in shared memory
 // (activation, scale and the decay's function applied on the way unless a pass before has applied them), the next
 // chunk's raw values are fetched into registers before the current chunk is worked on and written to the other
-// buffer afterwards.  A token's staged values are read one token ahead of the arithmetic that uses them.  Every
+// buffer afterwards.  A token's staged values are read one to three tokens ahead of the arithmetic that uses them.  Every
 // thread leaves one partial sum per token; after one barrier the block adds each token's R partial sums in the
 // order of r.  CH = 1 serves steps of single tokens: little shared memory, so that many blocks of a compute unit
 // have their state rows on the way at once.
-template <int PC, int NPT, bool BEFORE, int CH>
+template <int PC, int NPT, bool BEFORE, int CH, bool VEC = false>
 __global__ void __launch_bounds__(SCAN_THREADS)
 decay_scan_kernel(const ScanArgs a) {
   constexpr int R = SCAN_THREADS / PC;
@@ -77,7 +77,9 @@ decay_scan_kernel(const ScanArgs a) {
   constexpr int ROW = 3 * NP + PC;                  // staged values of a token: q | k | d | v
   constexpr int PER_BUF = CH * ROW;
   constexpr int LANES = SCAN_THREADS / CH;          // staging lanes of a token
-  constexpr int PER_TOK = (ROW + LANES - 1) / LANES;
+  constexpr int SV = VEC ? 4 : 1;                   // values a staging lane brings at once (VEC: 16-byte pieces)
+  constexpr int PER_TOK = (ROW / SV + LANES - 1) / LANES;
+  static_assert(!VEC || (NP % 4 == 0 && PC % 4 == 0), "16-byte pieces do not straddle q | k | d | v");
   extern __shared__ __attribute__((aligned(16))) float shared[];
   float* part = shared + 2 * PER_BUF;               // [chunk][R][PC]
   const int b = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * PC;
@@ -95,28 +97,35 @@ decay_scan_kernel(const ScanArgs a) {
   }
   const float head_decay = a.decay_kind == DECAY_PER_HEAD ? a.z[h] : 1.f;
   const int tl = tid / LANES, ln = tid % LANES;     // staging: token of the chunk, lane of its LANES
-  float raw[PER_TOK];
+  float raw[PER_TOK * SV];
   // element e of a token's staged row: [0, NP) q, [NP, 2NP) k, [2NP, 3NP) decay, then PC values of v
   auto fetch = [&](int c0) __attribute__((always_inline)) {
     const int tok = c0 + tl;
     const bool live = tok < end;
 #pragma unroll
     for (int i = 0; i < PER_TOK; ++i) {
-      const int e = ln + LANES * i;
-      float val = 0.f;
+      const int e = SV * (ln + LANES * i);
+      const float* src = nullptr;
       if (live && e < ROW) {
         if (e < 3 * NP) {
           const int which = e / NP, n = e % NP;
           if (n < N) {
-            if (which == 0) val = a.q[(size_t)tok * a.q_ld + h * N + n];
-            else if (which == 1) val = a.k[(size_t)tok * a.k_ld + h * N + n];
-            else if (a.decay_kind != DECAY_PER_HEAD) val = a.z[(size_t)tok * a.z_ld + h * N + n];
+            if (which == 0) src = a.q + (size_t)tok * a.q_ld + h * N + n;
+            else if (which == 1) src = a.k + (size_t)tok * a.k_ld + h * N + n;
+            else if (a.decay_kind != DECAY_PER_HEAD) src = a.z + (size_t)tok * a.z_ld + h * N + n;
           }
         } else if (p0 + e - 3 * NP < P) {
-          val = a.v[(size_t)tok * a.v_ld + h * P + p0 + e - 3 * NP];
+          src = a.v + (size_t)tok * a.v_ld + h * P + p0 + e - 3 * NP;
         }
       }
-      raw[i] = val;
+      if constexpr (VEC) {
+        // (N and P are multiples of four here: a piece lies inside its row or outside)
+        const scan_f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+        const scan_f32x4 val = src ? *reinterpret_cast<const scan_f32x4*>(src) : zero4;
+        raw[4 * i] = val.x, raw[4 * i + 1] = val.y, raw[4 * i + 2] = val.z, raw[4 * i + 3] = val.w;
+      } else {
+        raw[i] = src ? *src : 0.f;
+      }
     }
   };
   auto put = [&](int c0, float* buf) __attribute__((always_inline)) {
@@ -124,20 +133,30 @@ decay_scan_kernel(const ScanArgs a) {
     float* dst = buf + tl * ROW;
 #pragma unroll
     for (int i = 0; i < PER_TOK; ++i) {
-      const int e = ln + LANES * i;
-      if (e < ROW) {
-        float val = raw[i];
-        const int which = e < 3 * NP ? e / NP : 3;
-        if (which == 2) {
-          // tokens past the entry's end and rows past N: decay 1 on a state that takes nothing
-          if (!live || e % NP >= N) val = 1.f;
-          else if (a.decay_kind == DECAY_PER_HEAD) val = head_decay;
-          else if (a.decay_kind != DECAY_READY) val = decay_of(val, a.decay_kind, a.inv_tau);
-        } else {
-          if (a.silu_inputs) val = exact_silu(val);
-          if (which == 0) val *= a.q_scale;
+      const int e0 = SV * (ln + LANES * i);
+      if (e0 < ROW) {
+        const int which = e0 < 3 * NP ? e0 / NP : 3;
+        float val[SV];
+#pragma unroll
+        for (int j = 0; j < SV; ++j) {
+          float x = raw[SV * i + j];
+          if (which == 2) {
+            // tokens past the entry's end and rows past N: decay 1 on a state that takes nothing
+            if (!live || (e0 + j) % NP >= N) x = 1.f;
+            else if (a.decay_kind == DECAY_PER_HEAD) x = head_decay;
+            else if (a.decay_kind != DECAY_READY) x = decay_of(x, a.decay_kind, a.inv_tau);
+          } else {
+            if (a.silu_inputs) x = exact_silu(x);
+            if (which == 0) x *= a.q_scale;
+          }
+          val[j] = x;
         }
-        dst[e] = val;
+        if constexpr (VEC) {
+          const scan_f32x4 v4 = {val[0], val[1], val[2], val[3]};
+          *reinterpret_cast<scan_f32x4*>(dst + e0) = v4;
+        } else {
+          dst[e0] = val[0];
+        }
       }
     }
   };
@@ -192,9 +211,8 @@ decay_scan_kernel(const ScanArgs a) {
       TokenIn in;
       read_token(buf, 0, in);
       part[r * PC + p] = move_rows(in);
-    } else {
-      // two sets of registers take turns: a token's values are read while the token before is worked on (tokens
-      // past the entry's end were staged with k = 0 and a decay of one: they change nothing)
+    } else if constexpr (NPT > 8) {
+      // many rows a thread: two sets of registers take turns, a token's values are read one token ahead
       const int t_end = (n_tok + 1) & ~1;
       TokenIn in_a, in_b;
       read_token(buf, 0, in_a);
@@ -203,6 +221,26 @@ decay_scan_kernel(const ScanArgs a) {
         part[(t * R + r) * PC + p] = move_rows(in_a);
         read_token(buf, t + 2 < CH ? t + 2 : CH - 1, in_a);
         part[((t + 1) * R + r) * PC + p] = move_rows(in_b);
+      }
+    } else {
+      // four sets of registers take turns: a token's values are read three tokens ahead of the arithmetic that uses
+      // them, so that the reads' way through shared memory passes behind the work on the tokens before (tokens past
+      // the entry's end were staged with k = 0 and a decay of one: they change nothing)
+      const int t_end = (n_tok + 3) & ~3;
+      TokenIn in0, in1, in2, in3;
+      auto at = [](int t) __attribute__((always_inline)) { return t < CH ? t : CH - 1; };
+      read_token(buf, 0, in0);
+      read_token(buf, at(1), in1);
+      read_token(buf, at(2), in2);
+      for (int t = 0; t < t_end; t += 4) {
+        read_token(buf, at(t + 3), in3);
+        part[(t * R + r) * PC + p] = move_rows(in0);
+        read_token(buf, at(t + 4), in0);
+        part[((t + 1) * R + r) * PC + p] = move_rows(in1);
+        read_token(buf, at(t + 5), in1);
+        part[((t + 2) * R + r) * PC + p] = move_rows(in2);
+        read_token(buf, at(t + 6), in2);
+        part[((t + 3) * R + r) * PC + p] = move_rows(in3);
       }
     }
     shared_memory_barrier();
@@ -228,17 +266,17 @@ decay_scan_kernel(const ScanArgs a) {
   }
 }
 
-template <int PC, int NPT, bool BEFORE, int CH>
+template <int PC, int NPT, bool BEFORE, int CH, bool VEC = false>
 static int launch_decay_scan_as(const ScanArgs& a, int B_, hipStream_t stream) {
   constexpr int R = SCAN_THREADS / PC, NP = R * NPT;
   constexpr size_t need = (2 * (size_t)CH * (3 * NP + PC) + (size_t)CH * R * PC) * sizeof(float);
   static_assert(need <= 160 * 1024, "a block's staging fits the shared memory of a compute unit");
   if (need > 48 * 1024) {
-    const hipError_t e = hipFuncSetAttribute((const void*)decay_scan_kernel<PC, NPT, BEFORE, CH>,
+    const hipError_t e = hipFuncSetAttribute((const void*)decay_scan_kernel<PC, NPT, BEFORE, CH, VEC>,
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)need);
     if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL((decay_scan_kernel<PC, NPT, BEFORE, CH>), dim3(B_, a.heads, (a.P + PC - 1) / PC), dim3(SCAN_THREADS),
+  hipLaunchKernelGGL((decay_scan_kernel<PC, NPT, BEFORE, CH, VEC>), dim3(B_, a.heads, (a.P + PC - 1) / PC), dim3(SCAN_THREADS),
                      need, stream, a);
   ULLM_LAUNCH_CHECK();
 }
@@ -249,6 +287,18 @@ static int launch_decay_scan(const ScanArgs& a, int B_, bool single, hipStream_t
                               : launch_decay_scan_as<PC, NPT, true, SCAN_CHUNK>(a, B_, stream);
   return single ? launch_decay_scan_as<PC, NPT, false, 1>(a, B_, stream)
                 : launch_decay_scan_as<PC, NPT, false, SCAN_CHUNK>(a, B_, stream);
+}
+
+// Few blocks: longer chunks (fewer waits for the next chunk's values with nothing else to run meanwhile) and, where
+// the rows allow it, 16-byte pieces on their way into shared memory.
+template <int PC, int NPT, int CH>
+static int launch_decay_scan_few(const ScanArgs& a, int B_, hipStream_t stream) {
+  const bool vec = a.N % 4 == 0 && a.P % 4 == 0 && a.q_ld % 4 == 0 && a.k_ld % 4 == 0 && a.v_ld % 4 == 0 && a.z_ld % 4 == 0 &&
+                   ((uintptr_t)a.q | (uintptr_t)a.k | (uintptr_t)a.v | (uintptr_t)a.z) % 16 == 0;
+  if (vec) return a.before ? launch_decay_scan_as<PC, NPT, true, CH, true>(a, B_, stream)
+                           : launch_decay_scan_as<PC, NPT, false, CH, true>(a, B_, stream);
+  return a.before ? launch_decay_scan_as<PC, NPT, true, CH>(a, B_, stream)
+                  : launch_decay_scan_as<PC, NPT, false, CH>(a, B_, stream);
 }
 
 // max_len: the most tokens any entry brings (1: a step of single tokens).
@@ -274,6 +324,13 @@ extern "C" int ullm_decay_scan(const float* q, int q_ld, const float* k, int k_l
     if (N <= 32) SCAN_GO(64, 8);
     if (N <= 64) SCAN_GO(64, 16);
     SCAN_GO(64, 32);
+  }
+  // few blocks (one long prompt): slices of 8, so that twice as many compute units have a block
+  if (!single && (long long)B_ * heads * ((P + 15) / 16) < 256) {
+    if (N <= 32) return launch_decay_scan_few<8, 1, 32>(a, B_, stream);
+    if (N <= 64) return launch_decay_scan_few<8, 2, 32>(a, B_, stream);
+    if (N <= 128) return launch_decay_scan_few<8, 4, 32>(a, B_, stream);
+    return launch_decay_scan_few<8, 8, SCAN_CHUNK>(a, B_, stream);
   }
   if (N <= 16) SCAN_GO(16, 1);
   if (N <= 32) SCAN_GO(16, 2);

@@ -105,26 +105,45 @@ decay_scan_kernel(const ScanArgs a) {
 #pragma unroll
     for (int i = 0; i < PER_TOK; ++i) {
       const int e = SV * (ln + LANES * i);
-      const float* src = nullptr;
-      if (live && e < ROW) {
-        if (e < 3 * NP) {
-          const int which = e / NP, n = e % NP;
-          if (n < N) {
-            if (which == 0) src = a.q + (size_t)tok * a.q_ld + h * N + n;
-            else if (which == 1) src = a.k + (size_t)tok * a.k_ld + h * N + n;
-            else if (a.decay_kind != DECAY_PER_HEAD) src = a.z + (size_t)tok * a.z_ld + h * N + n;
+      if constexpr (VEC || CH == 1) {
+        // the address is chosen first and one load follows: the loads of a lane are all on their way before the
+        // first is waited for (a step of single tokens is made of such waits).  (With 16-byte pieces N and P are
+        // multiples of four: a piece lies inside its row or outside.)
+        const float* src = nullptr;
+        if (live && e < ROW) {
+          if (e < 3 * NP) {
+            const int which = e / NP, n = e % NP;
+            if (n < N) {
+              if (which == 0) src = a.q + (size_t)tok * a.q_ld + h * N + n;
+              else if (which == 1) src = a.k + (size_t)tok * a.k_ld + h * N + n;
+              else if (a.decay_kind != DECAY_PER_HEAD) src = a.z + (size_t)tok * a.z_ld + h * N + n;
+            }
+          } else if (p0 + e - 3 * NP < P) {
+            src = a.v + (size_t)tok * a.v_ld + h * P + p0 + e - 3 * NP;
           }
-        } else if (p0 + e - 3 * NP < P) {
-          src = a.v + (size_t)tok * a.v_ld + h * P + p0 + e - 3 * NP;
         }
-      }
-      if constexpr (VEC) {
-        // (N and P are multiples of four here: a piece lies inside its row or outside)
-        const scan_f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
-        const scan_f32x4 val = src ? *reinterpret_cast<const scan_f32x4*>(src) : zero4;
-        raw[4 * i] = val.x, raw[4 * i + 1] = val.y, raw[4 * i + 2] = val.z, raw[4 * i + 3] = val.w;
+        if constexpr (VEC) {
+          const scan_f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+          const scan_f32x4 val = src ? *reinterpret_cast<const scan_f32x4*>(src) : zero4;
+          raw[4 * i] = val.x, raw[4 * i + 1] = val.y, raw[4 * i + 2] = val.z, raw[4 * i + 3] = val.w;
+        } else {
+          raw[i] = src ? *src : 0.f;
+        }
       } else {
-        raw[i] = src ? *src : 0.f;
+        float val = 0.f;
+        if (live && e < ROW) {
+          if (e < 3 * NP) {
+            const int which = e / NP, n = e % NP;
+            if (n < N) {
+              if (which == 0) val = a.q[(size_t)tok * a.q_ld + h * N + n];
+              else if (which == 1) val = a.k[(size_t)tok * a.k_ld + h * N + n];
+              else if (a.decay_kind != DECAY_PER_HEAD) val = a.z[(size_t)tok * a.z_ld + h * N + n];
+            }
+          } else if (p0 + e - 3 * NP < P) {
+            val = a.v[(size_t)tok * a.v_ld + h * P + p0 + e - 3 * NP];
+          }
+        }
+        raw[i] = val;
       }
     }
   };
@@ -211,7 +230,7 @@ decay_scan_kernel(const ScanArgs a) {
       TokenIn in;
       read_token(buf, 0, in);
       part[r * PC + p] = move_rows(in);
-    } else if constexpr (NPT > 8) {
+    } else if constexpr (NPT > 4) {
       // many rows a thread: two sets of registers take turns, a token's values are read one token ahead
       const int t_end = (n_tok + 1) & ~1;
       TokenIn in_a, in_b;

@@ -553,11 +553,14 @@ def test_the_norm_of_the_outputs_with_gain_and_gate(parts, shared, gate_kind):
     act = plain.silu(z) if gate_kind == "silu" else torch.sigmoid(z)
     full_gain = gain.double().repeat(parts) if shared else gain.double()
     want = plain.unit_rms(o.double().view(T, parts, size), 1e-5).reshape(T, width) * full_gain * act
+    sliced = torch.randn(3, T, width, generator=g)
+    sliced[2] = o - sliced[0] - sliced[1]                # three slices whose sum is o
     for dtype in (torch.float32, torch.bfloat16):
-        got = ops.gated_unit_norm(o.to(DEV), wide.to(DEV)[:, 6:], gain.to(DEV), 1e-5, parts,
-                                  ops.GATE_SILU if gate_kind == "silu" else ops.GATE_SIGMOID, dtype)
-        assert got.dtype == dtype
-        assert (got.double().cpu() - want).abs().max() <= (2e-5 if dtype == torch.float32 else 2e-2) * want.abs().max()
+        for rows in (o, sliced):
+            got = ops.gated_unit_norm(rows.to(DEV), wide.to(DEV)[:, 6:], gain.to(DEV), 1e-5, parts,
+                                      ops.GATE_SILU if gate_kind == "silu" else ops.GATE_SIGMOID, dtype)
+            assert got.dtype == dtype and got.shape == (T, width)
+            assert (got.double().cpu() - want).abs().max() <= (2e-5 if dtype == torch.float32 else 2e-2) * want.abs().max()
 
 
 @pytest.mark.parametrize("S,H", [(1, 8), (2, 40), (3, 300), (4, 1024), (8, 33)])

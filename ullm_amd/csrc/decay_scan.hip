@@ -454,10 +454,18 @@ extern "C" int ullm_token_shift(const void* x, const float* mu, float* state, lo
 // one per column) and by silu or sigmoid of the gate's raw value g[t, c].  Parts of up to 1024 values: a wave per
 // (token, part), every lane's values in registers between the sum of squares and the scaling; longer parts: a block.
 #define NORM_PER_LANE 16
+// `slices` > 1: o is [slices, T, width] and a value is the sum of its slices, added in their order.
+__device__ __forceinline__ float sum_slices(const float* p, int slices, size_t stride) {
+  float v = p[0];
+  for (int s = 1; s < slices; ++s) v += p[(size_t)s * stride];
+  return v;
+}
+
 template <typename TO>
 __global__ void __launch_bounds__(256)
 gated_unit_norm_wave_kernel(const float* __restrict__ o, const float* __restrict__ g, int g_ld, const float* __restrict__ gain,
-                            int gain_len, float eps, int gate_kind, TO* __restrict__ out, int T_, int width, int parts) {
+                            int gain_len, float eps, int gate_kind, TO* __restrict__ out, int T_, int width, int parts,
+                            int slices) {
   const int lane = threadIdx.x % WAVE;
   const long long item = (long long)blockIdx.x * (256 / WAVE) + threadIdx.x / WAVE;
   if (item >= (long long)T_ * parts) return;
@@ -469,7 +477,7 @@ gated_unit_norm_wave_kernel(const float* __restrict__ o, const float* __restrict
 #pragma unroll
   for (int i = 0; i < NORM_PER_LANE; ++i) {
     const int c = lane + WAVE * i;
-    v[i] = c < size ? src[c] : 0.f;
+    v[i] = c < size ? sum_slices(src + c, slices, (size_t)T_ * width) : 0.f;
     z[i] = c < size ? g[(size_t)t * g_ld + part * size + c] : 0.f;
     sq += v[i] * v[i];
   }
@@ -488,27 +496,32 @@ gated_unit_norm_wave_kernel(const float* __restrict__ o, const float* __restrict
 template <typename TO>
 __global__ void __launch_bounds__(1024)
 gated_unit_norm_block_kernel(const float* __restrict__ o, const float* __restrict__ g, int g_ld, const float* __restrict__ gain,
-                             int gain_len, float eps, int gate_kind, TO* __restrict__ out, int width, int parts) {
+                             int gain_len, float eps, int gate_kind, TO* __restrict__ out, int T_, int width, int parts,
+                             int slices) {
   __shared__ float scratch[16];
   const int t = blockIdx.x / parts, part = blockIdx.x % parts;
   const int size = width / parts;
   const float* src = o + (size_t)t * width + (size_t)part * size;
+  const size_t stride = (size_t)T_ * width;
   float sq = 0.f;
-  for (int c = threadIdx.x; c < size; c += blockDim.x) sq += src[c] * src[c];
+  for (int c = threadIdx.x; c < size; c += blockDim.x) {
+    const float x = sum_slices(src + c, slices, stride);
+    sq += x * x;
+  }
   const float r = 1.f / sqrtf(block_sum(sq, scratch) / (float)size + eps);
   for (int c = threadIdx.x; c < size; c += blockDim.x) {
     const int col = part * size + c;
     const float z = g[(size_t)t * g_ld + col];
     const float gate = gate_kind == GATE_SIGMOID ? 1.f / (1.f + expf(-z)) : exact_silu(z);
-    st_f32(out + (size_t)t * width + col, src[c] * r * gain[col % gain_len] * gate);
+    st_f32(out + (size_t)t * width + col, sum_slices(src + c, slices, stride) * r * gain[col % gain_len] * gate);
   }
 }
 
 extern "C" int ullm_gated_unit_norm(const float* o, const float* g, int g_ld, const float* gain, int gain_len, float eps,
-                                    int gate_kind, void* out, int T_, int width, int parts, int out_dtype,
+                                    int gate_kind, void* out, int T_, int width, int parts, int slices, int out_dtype,
                                     hipStream_t stream) {
   if (T_ <= 0) return 0;
-  if (width < 1 || parts < 1 || width % parts || gain_len < 1 || width % gain_len) return ULLM_ERR_SHAPE;
+  if (width < 1 || parts < 1 || width % parts || gain_len < 1 || width % gain_len || slices < 1) return ULLM_ERR_SHAPE;
   if (gate_kind != GATE_SILU && gate_kind != GATE_SIGMOID) return ULLM_ERR_UNSUPPORTED;
   if (out_dtype != ULLM_F32 && out_dtype != ULLM_BF16) return ULLM_ERR_DTYPE;
   const int size = width / parts;
@@ -517,20 +530,20 @@ extern "C" int ullm_gated_unit_norm(const float* o, const float* g, int g_ld, co
     const dim3 grid((unsigned)((items + 3) / 4));
     if (out_dtype == ULLM_F32)
       hipLaunchKernelGGL(gated_unit_norm_wave_kernel<float>, grid, dim3(256), 0, stream, o, g, g_ld, gain, gain_len, eps,
-                         gate_kind, (float*)out, T_, width, parts);
+                         gate_kind, (float*)out, T_, width, parts, slices);
     else
       hipLaunchKernelGGL(gated_unit_norm_wave_kernel<bf16_t>, grid, dim3(256), 0, stream, o, g, g_ld, gain, gain_len, eps,
-                         gate_kind, (bf16_t*)out, T_, width, parts);
+                         gate_kind, (bf16_t*)out, T_, width, parts, slices);
   } else {
     int threads = 256;
     while (threads < size / 4 && threads < 1024) threads *= 2;
     const dim3 grid((unsigned)((long long)T_ * parts));
     if (out_dtype == ULLM_F32)
       hipLaunchKernelGGL(gated_unit_norm_block_kernel<float>, grid, dim3(threads), 0, stream, o, g, g_ld, gain, gain_len, eps,
-                         gate_kind, (float*)out, width, parts);
+                         gate_kind, (float*)out, T_, width, parts, slices);
     else
       hipLaunchKernelGGL(gated_unit_norm_block_kernel<bf16_t>, grid, dim3(threads), 0, stream, o, g, g_ld, gain, gain_len, eps,
-                         gate_kind, (bf16_t*)out, width, parts);
+                         gate_kind, (bf16_t*)out, T_, width, parts, slices);
   }
   ULLM_LAUNCH_CHECK();
 }

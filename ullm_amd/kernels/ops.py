@@ -636,8 +636,8 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.T
           and state_off + heads * key_dim * value_dim <= state.shape[1], "state must be float32 [slots, row] holding the heads' states")
     _i32(q_start, "q_start", n_entries + 1)
     _i32(entry_slot, "entry_slot", n_entries)
-    out = torch.empty((T, heads * value_dim), dtype=torch.float32, device=q.device)
     ll = ctypes.c_longlong
+    out = torch.empty((T, heads * value_dim), dtype=torch.float32, device=q.device)
     _check(build.load("decay_scan").ullm_decay_scan(
         _p(q), _c_int(q.stride(0)), _p(k), _c_int(k.stride(0)), _p(v), _c_int(v.stride(0)), _p(decay), _c_int(z_ld),
         _c_int(decay_kind), _c_float(tau), _p(bonus), _c_int(1 if silu_inputs else 0), _c_float(q_scale),
@@ -689,11 +689,14 @@ def token_shift(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, state_of
 
 def gated_unit_norm(o: torch.Tensor, gate: torch.Tensor, gain: torch.Tensor, eps: float, parts: int, gate_kind: int,
                     out_dtype: torch.dtype) -> torch.Tensor:
-    """Rows ``o`` (float32 [T, width]) cut into ``parts`` equal parts, each divided by its root mean square (eps inside
+    """Rows ``o`` (float32 [T, width], or [slices, T, width] whose slices are added first, in their order) cut into ``parts`` equal parts, each divided by its root mean square (eps inside
     the root), times ``gain`` (float32; as long as a part, shared by the parts, or as long as the row) and times
     silu or sigmoid (``gate_kind``) of ``gate`` (float32 [T, width], may be a column range of wider rows)."""
-    T, width = o.shape
-    _need(o.dtype == torch.float32 and o.is_contiguous(), "o must be contiguous float32")
+    slices = 1
+    if o.dim() == 3:
+        slices = o.shape[0]
+    T, width = o.shape[-2:]
+    _need(o.dtype == torch.float32 and o.is_contiguous(), "o must be contiguous float32 [T, width] or [slices, T, width]")
     _f32_rows(gate, "gate", T, width)
     _need(parts >= 1 and width % parts == 0, f"{width} values do not cut into {parts} equal parts")
     _need(gain.dtype == torch.float32 and gain.is_contiguous() and gain.numel() in (width // parts, width),
@@ -701,7 +704,7 @@ def gated_unit_norm(o: torch.Tensor, gate: torch.Tensor, gain: torch.Tensor, eps
     out = torch.empty((T, width), dtype=out_dtype, device=o.device)
     _check(build.load("decay_scan").ullm_gated_unit_norm(
         _p(o), _p(gate), _c_int(gate.stride(0)), _p(gain), _c_int(gain.numel()), _c_float(eps), _c_int(gate_kind), _p(out),
-        _c_int(T), _c_int(width), _c_int(parts), _c_int(_dt(out)), _stream()), "gated_unit_norm")
+        _c_int(T), _c_int(width), _c_int(parts), _c_int(slices), _c_int(_dt(out)), _stream()), "gated_unit_norm")
     return out
 
 

@@ -194,3 +194,13 @@ def test_the_plain_router_weights_and_window():
         total = s[t, 1] + s[t, other]
         want = sum(3.0 * s[t, e] / total * plain.gated_unit(h[t], w[f"m.e{e}.gate"], w[f"m.e{e}.up"], w[f"m.e{e}.down"]) for e in (1, other))
         assert torch.allclose(got[t], want, atol=1e-12)
+
+
+def test_a_file_may_hold_the_tensors_of_a_feed_forward_that_a_layer_does_not_have():
+    from ullm_amd.weights.loader import WeightError, check_against
+    _, model = build_model(CFG)
+    index = {d.name: ("f", tuple(d.shape), "BF16") for d in model.weight_decls() if d.alias_of is None}
+    extra = {"l2.norm2": ("f", (24,), "BF16"), "l2.hc2.mix": ("f", (3, 3), "BF16")}
+    check_against(model.weight_decls(), {**index, **extra}, frozenset(model.plan.unused_tensors))
+    with pytest.raises(WeightError, match="unexpected"):
+        check_against(model.weight_decls(), {**index, "l0.hc3.in": ("f", (3,), "BF16")}, frozenset(model.plan.unused_tensors))

@@ -48,9 +48,12 @@ def _mixer(m, prefix: str, H: int, eps: float) -> Choice:
 def kumudra_plan(cfg: KumudraConfig) -> ModelPlan:
     H, eps = cfg.hidden_size, cfg.norm_eps
     norm = lambda name: Choice("norm", "layernorm", dict(size=H, eps=eps, weight_name=name))      # noqa: E731
-    layers = []
+    layers, unused = [], []
     for i, L in enumerate(cfg.layers):
         p = f"l{i}"
+        if L.mlp is None:
+            # a layer without a feed-forward needs none of that sublayer's tensors; a file may hold them all the same
+            unused += [f"{p}.norm2", f"{p}.hc2.in", f"{p}.hc2.out", f"{p}.hc2.mix"]
         params = dict(hidden_size=H, streams=cfg.streams, mixer_norm=norm(f"{p}.norm1"), mixer=_mixer(L.mixer, f"{p}.mix", H, eps),
                       prefix=p, mult=cfg.residual_mult)
         f = L.mlp
@@ -77,6 +80,7 @@ def kumudra_plan(cfg: KumudraConfig) -> ModelPlan:
         vocab_size=cfg.vocab_size, hidden_size=H, embedding_weight="embed", layers=layers,
         final_norm=norm("final.norm"), head_weight="head", tie_head_to_embedding=True,
         embedding_scale=cfg.embedding_scale, streams=cfg.streams, run_order=order if len(order) != n else None,
+        unused_tensors=tuple(unused),
         init_std=0.05)
 
 

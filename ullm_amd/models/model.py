@@ -59,6 +59,9 @@ class ModelPlan:
     # and writes it; later entries with the same id only read it, so a layer can read the cache
     # another layer wrote.  Default: every layer once, cache id = layer index.
     run_order: Optional[List[Tuple[int, int]]] = None
+    # names a checkpoint may hold although this configuration has no use for them (a layer without a feed-forward
+    # whose export still wrote that sublayer's norm): not loaded, and no error
+    unused_tensors: Tuple[str, ...] = ()
     init_std: float = 0.02                   # random-weights mode
 
     def order(self) -> List[Tuple[int, int]]:

@@ -89,10 +89,11 @@ def merged_tensors(decls: List[WeightDecl]) -> Dict[str, MergedTensor]:
     return out
 
 
-def check_against(decls: List[WeightDecl], index) -> None:
+def check_against(decls: List[WeightDecl], index, unused=()) -> None:
     """One error that lists every missing tensor, every unexpected tensor and every wrong shape.
     A merged matrix may come as its pieces (the usual export) or whole under its merged name (the
-    reference takes both, ullm/layers/linear.py:359-379,473-485), not as a mixture."""
+    reference takes both, ullm/layers/linear.py:359-379,473-485), not as a mixture.  ``unused``: names a
+    checkpoint may hold although the model has no use for them (they are not loaded)."""
     declared = unique_decls(decls)
     merged = merged_tensors(decls)
     missing, wrong = [], []
@@ -110,7 +111,7 @@ def check_against(decls: List[WeightDecl], index) -> None:
         missing.append(f"  {name}  expected shape {list(d.shape)}")
     unexpected = []
     for n in sorted(index):
-        if n in declared or n.endswith(IGNORABLE_SUFFIXES):
+        if n in declared or n.endswith(IGNORABLE_SUFFIXES) or n in unused:
             continue
         if n in merged:
             m = merged[n]
@@ -151,7 +152,7 @@ def load_weights(model, model_dir: str, env: PartEnv) -> None:
     copied from the file straight into its rows, so nothing is held twice on the device."""
     decls = model.weight_decls()
     index = checkpoint_index(model_dir)
-    check_against(decls, index)
+    check_against(decls, index, frozenset(getattr(model.plan, "unused_tensors", ())))
     declared = unique_decls(decls)
     merged = merged_tensors(decls)
     # what to read from each file: (name in the file, declaration it fills or None for a whole merged matrix)

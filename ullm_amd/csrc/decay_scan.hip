@@ -81,7 +81,8 @@ decay_scan_kernel(const ScanArgs a) {
   constexpr int PER_TOK = (ROW / SV + LANES - 1) / LANES;
   static_assert(!VEC || (NP % 4 == 0 && PC % 4 == 0), "16-byte pieces do not straddle q | k | d | v");
   extern __shared__ __attribute__((aligned(16))) float shared[];
-  float* part = shared + 2 * PER_BUF;               // [chunk][R][PC]
+  constexpr int PART = R * PC + (PC < 64 ? PC : 0);   // a token's partial sums, padded: the tokens of a wave's lanes in other banks
+  float* part = shared + 2 * PER_BUF;               // [chunk][PART]
   const int b = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * PC;
   const int tid = threadIdx.x, p = tid % PC, r = tid / PC;
   const int N = a.N, P = a.P;
@@ -237,42 +238,45 @@ decay_scan_kernel(const ScanArgs a) {
       read_token(buf, 0, in_a);
       for (int t = 0; t < t_end; t += 2) {
         read_token(buf, t + 1, in_b);
-        part[(t * R + r) * PC + p] = move_rows(in_a);
+        part[t * PART + r * PC + p] = move_rows(in_a);
         read_token(buf, t + 2 < CH ? t + 2 : CH - 1, in_a);
-        part[((t + 1) * R + r) * PC + p] = move_rows(in_b);
+        part[(t + 1) * PART + r * PC + p] = move_rows(in_b);
       }
     } else {
       // four sets of registers take turns: a token's values are read three tokens ahead of the arithmetic that uses
       // them, so that the reads' way through shared memory passes behind the work on the tokens before (tokens past
       // the entry's end were staged with k = 0 and a decay of one: they change nothing)
-      const int t_end = (n_tok + 3) & ~3;
+      // (the whole chunk is walked, so that the loop unrolls and every address in shared memory is a constant)
       TokenIn in0, in1, in2, in3;
       auto at = [](int t) __attribute__((always_inline)) { return t < CH ? t : CH - 1; };
       read_token(buf, 0, in0);
       read_token(buf, at(1), in1);
       read_token(buf, at(2), in2);
-      for (int t = 0; t < t_end; t += 4) {
+#pragma unroll
+      for (int t = 0; t < CH; t += 4) {
         read_token(buf, at(t + 3), in3);
-        part[(t * R + r) * PC + p] = move_rows(in0);
+        part[t * PART + r * PC + p] = move_rows(in0);
         read_token(buf, at(t + 4), in0);
-        part[((t + 1) * R + r) * PC + p] = move_rows(in1);
+        part[(t + 1) * PART + r * PC + p] = move_rows(in1);
         read_token(buf, at(t + 5), in1);
-        part[((t + 2) * R + r) * PC + p] = move_rows(in2);
+        part[(t + 2) * PART + r * PC + p] = move_rows(in2);
         read_token(buf, at(t + 6), in2);
-        part[((t + 3) * R + r) * PC + p] = move_rows(in3);
+        part[(t + 3) * PART + r * PC + p] = move_rows(in3);
       }
     }
+    // the next chunk goes to the other buffer before this chunk's results are stored: the wait for its loads then
+    // does not also wait for those stores (loads and stores are counted together, in order)
+    if (more) put(c0 + CH, shared + (1 - turn) * PER_BUF);
     shared_memory_barrier();
     for (int e = tid; e < n_tok * PC; e += SCAN_THREADS) {
       const int t = e / PC, pp = e % PC;
       if (p0 + pp < P) {
         float sum = 0.f;
 #pragma unroll
-        for (int i = 0; i < R; ++i) sum += part[(t * R + i) * PC + pp];
+        for (int i = 0; i < R; ++i) sum += part[t * PART + i * PC + pp];
         a.out[(size_t)(c0 + t) * a.heads * P + h * P + p0 + pp] = sum;
       }
     }
-    if (more) put(c0 + CH, shared + (1 - turn) * PER_BUF);
     shared_memory_barrier();
     turn = 1 - turn;
   }
@@ -288,7 +292,7 @@ decay_scan_kernel(const ScanArgs a) {
 template <int PC, int NPT, bool BEFORE, int CH, bool VEC = false>
 static int launch_decay_scan_as(const ScanArgs& a, int B_, hipStream_t stream) {
   constexpr int R = SCAN_THREADS / PC, NP = R * NPT;
-  constexpr size_t need = (2 * (size_t)CH * (3 * NP + PC) + (size_t)CH * R * PC) * sizeof(float);
+  constexpr size_t need = (2 * (size_t)CH * (3 * NP + PC) + (size_t)CH * (R * PC + (PC < 64 ? PC : 0))) * sizeof(float);
   static_assert(need <= 160 * 1024, "a block's staging fits the shared memory of a compute unit");
   if (need > 48 * 1024) {
     const hipError_t e = hipFuncSetAttribute((const void*)decay_scan_kernel<PC, NPT, BEFORE, CH, VEC>,
@@ -300,20 +304,32 @@ static int launch_decay_scan_as(const ScanArgs& a, int B_, hipStream_t stream) {
   ULLM_LAUNCH_CHECK();
 }
 
+// 16-byte pieces on the way into shared memory: rows and offsets that are multiples of four values
+static bool scan_rows_in_pieces(const ScanArgs& a) {
+  const bool raw_decays = a.decay_kind != DECAY_PER_HEAD;       // else z holds the heads' constants and is not staged
+  return a.N % 4 == 0 && a.P % 4 == 0 && a.q_ld % 4 == 0 && a.k_ld % 4 == 0 && a.v_ld % 4 == 0 &&
+         ((uintptr_t)a.q | (uintptr_t)a.k | (uintptr_t)a.v) % 16 == 0 &&
+         (!raw_decays || (a.z_ld % 4 == 0 && (uintptr_t)a.z % 16 == 0));
+}
+
 template <int PC, int NPT>
 static int launch_decay_scan(const ScanArgs& a, int B_, bool single, hipStream_t stream) {
-  if (a.before) return single ? launch_decay_scan_as<PC, NPT, true, 1>(a, B_, stream)
-                              : launch_decay_scan_as<PC, NPT, true, SCAN_CHUNK>(a, B_, stream);
-  return single ? launch_decay_scan_as<PC, NPT, false, 1>(a, B_, stream)
-                : launch_decay_scan_as<PC, NPT, false, SCAN_CHUNK>(a, B_, stream);
+  if (single) return a.before ? launch_decay_scan_as<PC, NPT, true, 1>(a, B_, stream)
+                              : launch_decay_scan_as<PC, NPT, false, 1>(a, B_, stream);
+  if constexpr ((SCAN_THREADS / PC * NPT) % 4 == 0) {
+    if (scan_rows_in_pieces(a))
+      return a.before ? launch_decay_scan_as<PC, NPT, true, SCAN_CHUNK, true>(a, B_, stream)
+                      : launch_decay_scan_as<PC, NPT, false, SCAN_CHUNK, true>(a, B_, stream);
+  }
+  return a.before ? launch_decay_scan_as<PC, NPT, true, SCAN_CHUNK>(a, B_, stream)
+                  : launch_decay_scan_as<PC, NPT, false, SCAN_CHUNK>(a, B_, stream);
 }
 
 // Few blocks: longer chunks (fewer waits for the next chunk's values with nothing else to run meanwhile) and, where
 // the rows allow it, 16-byte pieces on their way into shared memory.
 template <int PC, int NPT, int CH>
 static int launch_decay_scan_few(const ScanArgs& a, int B_, hipStream_t stream) {
-  const bool vec = a.N % 4 == 0 && a.P % 4 == 0 && a.q_ld % 4 == 0 && a.k_ld % 4 == 0 && a.v_ld % 4 == 0 && a.z_ld % 4 == 0 &&
-                   ((uintptr_t)a.q | (uintptr_t)a.k | (uintptr_t)a.v | (uintptr_t)a.z) % 16 == 0;
+  const bool vec = scan_rows_in_pieces(a);
   if (vec) return a.before ? launch_decay_scan_as<PC, NPT, true, CH, true>(a, B_, stream)
                            : launch_decay_scan_as<PC, NPT, false, CH, true>(a, B_, stream);
   return a.before ? launch_decay_scan_as<PC, NPT, true, CH>(a, B_, stream)

@@ -192,21 +192,22 @@ def dovisun_config(shape):
 
 
 # Kumudra at a design shape: the same width; four layers passed twice, so eight layer runs a token as the other stacks
-# have, over two copies of the residual stream: gated linear attention (keys of half the head size) with the dense
-# feed-forward, two lightning layers and one layer of windowed attention (the other stacks' heads, a window of 1024 keys,
+# have, over two copies of the residual stream: two lightning layers, gated linear attention (keys of half the head
+# size) with the dense feed-forward, and one layer of windowed attention (the other stacks' heads, a window of 1024 keys,
 # half of each head rotated) beside time mixing (heads of 64), these three with routed feed-forwards of as many columns
 # a token as the dense one (top 4 of 32 experts of a sixth of it).
 def kumudra_config(shape):
     (W, H, G, D, F, L), _ = DESIGN_SHAPES[shape]
     moe = dict(kind="moe", router=dict(experts=32, top=4, scale=2.5), expert=dict(ff=F // 6))
+    gla = dict(type="gla", mixer=dict(heads=H, dim=D // 2, vdim=D, tau=8.0), mlp=dict(kind="dense", ff=F))
     lightning = dict(heads=H, dim=D, vdim=D, decay=[1.0 - 2.0 ** (-5.0 - 4.0 * h / max(1, H - 1)) for h in range(H)])
     left = dict(heads=H, kv_heads=G, dim=D, vdim=D, scale=D ** -0.5, mask=dict(size=1024),
-                rot=dict(base=500000.0, dims=D // 2, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)))
-    layers = [dict(type="gla", mixer=dict(heads=H, dim=D // 2, vdim=D, tau=16.0), mlp=dict(kind="dense", ff=F)),
-              dict(type="lightning", mixer=lightning, mlp=moe), dict(type="lightning", mixer=lightning, mlp=moe),
-              dict(type="parallel", mlp=moe, mixer=dict(left=left, right=dict(heads=W // 64, dim=64), left_scale=0.6, right_scale=0.9))]
+                rot=dict(base=500000.0, dims=D // 2, scaling=dict(factor=4.0, low=1.0, high=8.0, original=8192)))
+    layers = [dict(type="lightning", mixer=lightning, mlp=moe), gla,
+              dict(type="parallel", mlp=moe, mixer=dict(left=left, right=dict(heads=W // 64, dim=64), left_scale=0.5, right_scale=1.0)),
+              dict(type="lightning", mixer=lightning, mlp=moe)]
     return dict(architecture="Kumudra", vocab=DESIGN_VOCAB, width=W, norm=dict(eps=1e-5), layers=layers, streams=2,
-                residual_mult=0.7, embedding=dict(scale=1.0), loop=dict(start=0, stop=4, times=max(1, L // 4)))
+                residual_mult=0.5, embedding=dict(scale=1.0), loop=dict(start=0, stop=4, times=max(1, L // 4)))
 
 
 def design_run(args):

@@ -31,7 +31,7 @@ def light(heads, dim, vdim, decay, mlp=None):
     return dict(type="lightning", mixer=dict(heads=heads, dim=dim, vdim=vdim, decay=list(decay)), mlp=mlp)
 
 
-def par(heads, kv, dim, vdim, scale, window=None, rot=None, scaling=None, base=10000.0, right=(2, 8), scales=(0.6, 0.9), mlp=None, rank=4):
+def par(heads, kv, dim, vdim, scale, window=None, rot=None, scaling=None, base=10000.0, right=(2, 8), scales=(0.5, 1.1), mlp=None, rank=4):
     left = dict(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, scale=scale)
     if window:
         left["mask"] = dict(size=window)
@@ -63,7 +63,7 @@ def config(width, vocab, layers, streams=2, loop=None, eps=1e-5, scale=None, mul
 
 
 # A: every kind of layer, the two middle ones passed twice, three copies of the stream
-CFG_A = config(48, 131, [par(6, 2, 16, 24, 0.3, window=21, rot=8, scaling=(4.0, 1.0, 4.0, 64), right=(3, 8), mlp=moe(6, 2, 20, 1.5)),
+CFG_A = config(48, 131, [par(6, 2, 16, 24, 0.3, window=21, rot=8, scaling=(4.0, 1.0, 4.0, 64), right=(3, 8), mlp=moe(6, 2, 20, 1.75)),
                          gla(3, 8, 16, 8.0, mlp=dense(72)), light(2, 16, 8, (0.6, 0.995), mlp=moe(5, 3, 12, 0.8)),
                          gla(2, 12, 12, 2.0, mlp=None)], streams=3, loop=(1, 3, 2), scale=0.7, mult=0.6)
 # B: values that make things equal or one: one copy of the stream without coefficients in the file, no loop, no scale, no
@@ -77,7 +77,7 @@ CFG_B = config(40, 97, [par(3, 3, 6, 10, 0.5, right=(1, 6), scales=(1.0, 1.0), m
 # C: head sizes of 128 and 64 in the attention, a window shorter than a page, recurrences with 64, 128 and 192 key channels,
 # four copies, the whole stack passed three times
 CFG_C = config(64, 211, [par(4, 2, 128, 64, 0.09, window=5, rot=32, scaling=(8.0, 1.0, 2.0, 32), base=100.0, right=(2, 64), mlp=moe(8, 2, 16, 1.2)),
-                         gla(2, 128, 128, 16.0, mlp=None), light(1, 192, 32, (0.97,), mlp=dense(80))], streams=4, loop=(0, 3, 3),
+                         gla(2, 128, 128, 12.0, mlp=None), light(1, 192, 32, (0.97,), mlp=dense(80))], streams=4, loop=(0, 3, 3),
                scale=1.3, mult=0.4)
 # W: attention scores of many units under a window of 33 keys, beside a weak recurrent half
 CFG_W = config(32, 64, [par(2, 1, 16, 16, 3.0, window=33, rot=8, right=(1, 4), scales=(1.0, 0.05), mlp=None)], streams=2, scale=1.0)
@@ -87,7 +87,7 @@ CFG_GLA = config(32, 64, [gla(2, 16, 8, 4.0, mlp=None)], streams=2)
 CFG_LIGHT = config(32, 64, [light(2, 8, 16, (0.8, 0.999), mlp=None)], streams=2)
 CFG_PAR = config(32, 64, [par(4, 2, 8, 8, 0.35, window=12, rot=4, mlp=None)], streams=2)
 CFG_DENSE = config(32, 64, [gla(1, 8, 8, 4.0, mlp=dense(40))], streams=3)
-CFG_MOE = config(32, 64, [gla(1, 8, 8, 4.0, mlp=moe(7, 3, 8, 1.5))], streams=3)
+CFG_MOE = config(32, 64, [gla(1, 8, 8, 4.0, mlp=moe(7, 3, 8, 1.25))], streams=3)
 
 MODELS = {"A": (CFG_A, 1), "B": (CFG_B, 2), "C": (CFG_C, 3), "W": (CFG_W, 4), "M": (CFG_M, 5), "gla": (CFG_GLA, 6),
           "light": (CFG_LIGHT, 7), "par": (CFG_PAR, 8), "dense": (CFG_DENSE, 9), "moe": (CFG_MOE, 10)}
@@ -138,12 +138,14 @@ def oracle_and_gaps(models, name, toks):
     return _oracle_cache[key]
 
 
-# bfloat16 bounds (median, 85th of 100 rows, largest clear row).  A router that reads a rounded input picks another
-# expert where two choice scores lie closer than rounding moves them: such a row moves as a whole, and what it leaves in
-# the state moves the rows behind it a little.  So most rows are held to rounding, and every row whose own choices are
-# CLOSE_CALL or more apart to a bound that a lost key or a stale slot exceeds.
+# bfloat16 bounds (median, 85th of 100 rows, largest row).  A router that reads a rounded input picks another expert
+# where two choice scores lie closer than rounding moves them: such a row moves as a whole, and so does every row behind
+# it, which sees that token through the layers' states.  So the rows ahead of the first close call (a gap below
+# CLOSE_CALL between the last taken and the first left choice score, in the 64-bit implementation) are held to rounding
+# and to a bound that a lost key, a stale slot or a state one token off exceeds; the rows behind it only to a bound that
+# a wrong state or window exceeds by far on most rows (the median).
 BF16_BOUNDS = {"C": (4e-2, 1e-1, 0.3)}
-CLOSE_CALL = 0.02
+CLOSE_CALL = 0.01
 
 
 def close(got, want, dtype, name="", gaps=None):
@@ -151,14 +153,18 @@ def close(got, want, dtype, name="", gaps=None):
     if dtype == "float32":
         assert err.max() <= REL[dtype], f"max {err.max():.3e} at row {int(err.argmax())}"
         return
+    assert np.isfinite(got).all()
     mid, most, top = BF16_BOUNDS.get(name, (2e-2, 4e-2, 0.3))
-    clear = err if gaps is None else err[gaps >= CLOSE_CALL]
+    calls = np.nonzero(gaps < CLOSE_CALL)[0] if gaps is not None else []
+    sharp = err[:int(calls[0])] if len(calls) else err
+    if len(sharp) >= 8:
+        assert np.median(sharp) <= mid and np.quantile(sharp, 0.85) <= most, \
+            f"median {np.median(sharp):.3e}, 85th {np.quantile(sharp, 0.85):.3e} over {len(sharp)} rows"
+    elif len(sharp):
+        assert np.median(sharp) <= most, f"median {np.median(sharp):.3e}"
+    assert not len(sharp) or sharp.max() <= top, f"max {sharp.max():.3e} at row {int(sharp.argmax())}"
     if len(err) >= 8:
-        assert np.median(err) <= mid and np.quantile(err, 0.85) <= most, \
-            f"median {np.median(err):.3e}, 85th {np.quantile(err, 0.85):.3e}"
-    elif len(clear):
-        assert np.median(clear) <= most, f"median {np.median(clear):.3e}"
-    assert not len(clear) or clear.max() <= top, f"max {clear.max():.3e} at row {int(err.argmax())}"
+        assert np.median(err) <= 0.25, f"median {np.median(err):.3e} behind a close call"
 
 
 def agree(models, name, toks, got, dtype, rows=None):

@@ -33,7 +33,7 @@ def drawn_layer(rng):
     kind = rng.random()
     if kind < 0.3:
         mixer = dict(heads=rng.choice([1, 2, 3, 4, 8]), dim=rng.choice([4, 6, 8, 16, 32, 40, 64, 128]),
-                     vdim=rng.choice([4, 10, 16, 32, 64, 72, 128]), tau=rng.choice([1.0, 4.0, 16.0]), rank=rng.choice([1, 4, 16, 24]))
+                     vdim=rng.choice([4, 10, 16, 32, 64, 72, 128]), tau=rng.choice([1.0, 4.0, 12.0]), rank=rng.choice([1, 4, 16, 24]))
         return dict(type="gla", mixer=mixer, mlp=drawn_mlp(rng))
     if kind < 0.6:
         heads = rng.choice([1, 2, 3, 4, 8])
@@ -47,14 +47,14 @@ def drawn_layer(rng):
     if rng.random() < 0.8:
         left["mask"] = dict(size=rng.choice([1, 2, 5, 16, 17, 33, 64, 100]))
     if rng.random() < 0.8:
-        left["rot"] = dict(base=rng.choice([100.0, 10000.0, 250000.0]), dims=rng.choice([d for d in (2, 4, 8, 16, 32, 64, dim) if d <= dim]))
+        left["rot"] = dict(base=rng.choice([100.0, 10000.0, 500000.0]), dims=rng.choice([d for d in (2, 4, 8, 16, 32, 64, dim) if d <= dim]))
         if rng.random() < 0.7:
             low = rng.choice([1.0, 2.0])
             left["rot"]["scaling"] = dict(factor=rng.choice([1.0, 2.0, 8.0, 32.0]), low=low, high=low * rng.choice([2.0, 4.0]),
                                           original=rng.choice([16, 64, 512, 4096]))
     right = dict(heads=rng.choice([1, 2, 3, 6]), dim=rng.choice([4, 6, 8, 16, 32, 64]), rank=rng.choice([1, 4, 16, 20]))
-    return dict(type="parallel", mlp=drawn_mlp(rng), mixer=dict(left=left, right=right, left_scale=rng.choice([1.0, 0.6, 0.3]),
-                                                               right_scale=rng.choice([1.0, 0.9, 1.4])))
+    return dict(type="parallel", mlp=drawn_mlp(rng), mixer=dict(left=left, right=right, left_scale=rng.choice([1.0, 0.55, 0.3]),
+                                                               right_scale=rng.choice([1.0, 0.8, 1.4])))
 
 
 def drawn_config(rng):
@@ -67,7 +67,7 @@ def drawn_config(rng):
     if rng.random() < 0.7:
         cfg["embedding"] = dict(scale=rng.choice([0.5, 3.0, 11.0]))
     if rng.random() < 0.7:
-        cfg["residual_mult"] = rng.choice([0.3, 0.7, 1.5])
+        cfg["residual_mult"] = rng.choice([0.3, 0.65, 1.5])
     return cfg
 
 

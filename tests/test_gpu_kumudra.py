@@ -451,7 +451,7 @@ def _entries(lens, device):
     return to(token_entry), to(q_start), to(slots)
 
 
-@pytest.mark.parametrize("heads,N,P", [(1, 1, 1), (3, 6, 10), (2, 32, 64), (4, 64, 16), (2, 128, 128), (1, 200, 24), (2, 17, 33)])
+@pytest.mark.parametrize("heads,N,P", [(1, 1, 1), (3, 6, 10), (2, 32, 64), (4, 64, 16), (2, 128, 128), (1, 200, 24), (2, 17, 33), (1, 384, 20)])
 @pytest.mark.parametrize("kind", ["per_head", "sigmoid_root", "exp_exp_bonus"])
 @pytest.mark.parametrize("ahead", [False, True])
 def test_the_recurrence_alone(heads, N, P, kind, ahead):

@@ -346,7 +346,7 @@ extern "C" int ullm_decay_scan(const float* q, int q_ld, const float* k, int k_l
                                const int* q_start, const int* entry_slot, float* out, int B_, int heads, int N, int P,
                                int write_state, int max_len, hipStream_t stream) {
   if (B_ <= 0) return 0;
-  if (heads <= 0 || N <= 0 || P <= 0 || N > 256) return ULLM_ERR_SHAPE;
+  if (heads <= 0 || N <= 0 || P <= 0 || N > 512) return ULLM_ERR_SHAPE;
   if (decay_kind < DECAY_PER_HEAD || decay_kind > DECAY_READY || z == nullptr) return ULLM_ERR_UNSUPPORTED;
   if (decay_kind == DECAY_SIGMOID_ROOT && !(tau > 0.f)) return ULLM_ERR_UNSUPPORTED;
   ScanArgs a;
@@ -364,7 +364,7 @@ extern "C" int ullm_decay_scan(const float* q, int q_ld, const float* k, int k_l
     SCAN_GO(64, 32);
   }
   // few blocks (one long prompt): slices of 8, so that twice as many compute units have a block
-  if (!single && (long long)B_ * heads * ((P + 15) / 16) < 256) {
+  if (!single && N <= 256 && (long long)B_ * heads * ((P + 15) / 16) < 256) {
     if (N <= 32) return launch_decay_scan_few<8, 1, 32>(a, B_, stream);
     if (N <= 64) return launch_decay_scan_few<8, 2, 32>(a, B_, stream);
     if (N <= 128) return launch_decay_scan_few<8, 4, 32>(a, B_, stream);
@@ -374,7 +374,8 @@ extern "C" int ullm_decay_scan(const float* q, int q_ld, const float* k, int k_l
   if (N <= 32) SCAN_GO(16, 2);
   if (N <= 64) SCAN_GO(16, 4);
   if (N <= 128) SCAN_GO(16, 8);
-  SCAN_GO(16, 16);
+  if (N <= 256) SCAN_GO(16, 16);
+  SCAN_GO(16, 32);
 #undef SCAN_GO
 }
 

@@ -597,7 +597,7 @@ def weighted_sum(x: torch.Tensor, y: torch.Tensor, a: float, b: float) -> torch.
 
 DECAY_PER_HEAD, DECAY_SIGMOID_ROOT, DECAY_EXP_EXP, DECAY_READY = 0, 1, 2, 3      # how a recurrence's decays come about
 GATE_SILU, GATE_SIGMOID = 0, 1
-DECAY_SCAN_MAX_KEYS = 256
+DECAY_SCAN_MAX_KEYS = 512
 
 
 def _f32_rows(t: torch.Tensor, name: str, T: int, cols: int) -> None:

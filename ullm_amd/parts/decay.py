@@ -54,6 +54,13 @@ class _DecayMixer(Mixer):
     def _rows(cache: LayerCache) -> torch.Tensor:
         return cache.state.view(cache.state.shape[0], -1)
 
+    @staticmethod
+    def _ahead(x: torch.Tensor, ctx: StepContext) -> bool:
+        """Whether a pass of its own applies the inputs' functions ahead of the recurrence: in steps of many tokens
+        with portions of prompts (the recurrence's blocks, one per slice of value channels, would each apply them to a
+        whole chunk again); a step of single tokens leaves them to the recurrence, a launch fewer."""
+        return x.shape[0] >= ops.DECAY_PREPARE_FROM and ctx.max_q_len > 1
+
 
 @register_part("mixer", "gated_linear_attention")
 class GatedLinearAttention(_DecayMixer):
@@ -93,7 +100,7 @@ class GatedLinearAttention(_DecayMixer):
         z = linear(linear(x, self.w_a1, out_dtype=torch.float32), self.w_a2, self.b_a2, out_dtype=torch.float32)
         qk, inner = self.qk, self.inner
         kind = ops.DECAY_SIGMOID_ROOT
-        if x.shape[0] >= ops.DECAY_PREPARE_FROM:
+        if self._ahead(x, ctx):
             # many tokens: the decays' function is applied once per value ahead of the recurrence, not by each of its blocks
             ops.decay_prepare(None, z, kind, self.tau)
             kind = ops.DECAY_READY
@@ -135,7 +142,7 @@ class LightningAttention(_DecayMixer):
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
         proj = linear(x, self.w_in, out_dtype=torch.float32)                        # q | k | v | g
         qk, inner = self.qk, self.inner
-        ahead = x.shape[0] >= ops.DECAY_PREPARE_FROM
+        ahead = self._ahead(x, ctx)
         if ahead:
             ops.decay_prepare(proj[:, :2 * qk + inner])              # silu of q | k | v once per value
         o = ops.decay_scan(proj[:, :qk], proj[:, qk:2 * qk], proj[:, 2 * qk:2 * qk + inner], self.decay, ops.DECAY_PER_HEAD,
@@ -188,7 +195,7 @@ class TimeMix(_DecayMixer):
         g = linear(blends[3], self.w_g, out_dtype=f32)
         z = linear(linear(blends[4], self.w_w1, out_dtype=f32, act=ops.ACT_TANH), self.w_w2, self.w0, out_dtype=f32)
         kind = ops.DECAY_EXP_EXP
-        if x.shape[0] >= ops.DECAY_PREPARE_FROM:
+        if self._ahead(x, ctx):
             ops.decay_prepare(None, z, kind)
             kind = ops.DECAY_READY
         o = ops.decay_scan(r, k, v, z, kind, rows, self.carry, ctx.q_start, ctx.entry_slot, ctx.num_entries,
